@@ -1,11 +1,12 @@
 from .base import ConfigError, ModelConfig, read_config_json
 from .llama import LlamaConfig
+from .nusilix import NusilixConfig, NusilixLayer
 from .registry import (Architecture, register_architecture, unregister_architecture,
                        registered_architectures, resolve_architecture, config_from_dict,
                        load_config)
 
 __all__ = [
-    "ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "Architecture",
+    "ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "NusilixConfig", "NusilixLayer", "Architecture",
     "register_architecture", "unregister_architecture", "registered_architectures",
     "resolve_architecture", "config_from_dict", "load_config",
 ]

@@ -44,6 +44,8 @@ def registered_architectures():
 
 def resolve_architecture(raw: dict, where: str = "config.json") -> Architecture:
     archs = raw.get("architectures")
+    if not (isinstance(archs, list) and archs) and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]          # some configurations name the one architecture directly
     if isinstance(archs, list) and archs:
         name = archs[0]
         if name in _ARCHITECTURES:

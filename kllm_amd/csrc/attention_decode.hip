@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window,
-    float scale, int head_tiles, const int* __restrict__ token_list) {
+    float scale, const float* __restrict__ slopes, int head_tiles, const int* __restrict__ token_list) {
   constexpr int hd = 16 * HDT;
   constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
   constexpr int kDecodeAhead = decode_ahead(HDT);
@@ -84,6 +84,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   const bool head_ok = head_in_group < G;
   const int head = kvh * G + (head_ok ? head_in_group : 0);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const float slope = (slopes && head_ok) ? slopes[head] : 0.f;   // a bias that grows with the distance to the key
 
   bf16x8 qb[KS];
 #pragma unroll
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = kb + 16 * u + 4 * g + i;
         const bool ok = cur.live[u] && key >= start && key < len;
-        s[u][i] = ok ? s[u][i] * scale : -INFINITY;
+        s[u][i] = ok ? s[u][i] * scale - slope * (float)(len - 1 - key) : -INFINITY;
         tmax = fmaxf(tmax, s[u][i]);
       }
     tmax = group4_max(tmax);
@@ -281,7 +282,7 @@ template <int HDT, int W>
 static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out, float* part,
                          const void* cache, const int* positions, const int* span_of_token,
                          const int* block_table, int max_pages, int page_size, int H, int KV, int window,
-                         float scale, int head_tiles, const int* token_list) {
+                         float scale, const float* slopes, int head_tiles, const int* token_list) {
   const int heads = H / KV < 16 ? H / KV : 16;
   const size_t lds = (size_t)W * heads * (16 * HDT + 4) * sizeof(float);
   static int raised = 0;
@@ -294,7 +295,7 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
   }
   hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
-                     block_table, max_pages, page_size, H, KV, window, scale, head_tiles, token_list);
+                     block_table, max_pages, page_size, H, KV, window, scale, slopes, head_tiles, token_list);
   return 0;
 }
 
@@ -391,7 +392,7 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
 static int attn_decode_run(const char* who, const void* q, void* out, float* part, long part_floats,
                            const void* cache, const int* positions, const int* span_of_token,
                            const int* block_table, int max_pages, int page_size, int n, int H, int KV,
-                           int hd, int window, float scale, int nslices, int dtype,
+                           int hd, int window, float scale, const float* slopes, int nslices, int dtype,
                            const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
                "%s: null pointer", who);
@@ -405,7 +406,7 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
     KLLM_REQUIRE(H <= 65535, "%s: too many heads for the grid", who);
     KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "%s: bad token list", who);
     return attn_f32_decode((const float*)q, (float*)out, part, (const float*)cache, positions, span_of_token,
-                           block_table, max_pages, page_size, H, KV, hd, window, scale, nslices, token_list,
+                           block_table, max_pages, page_size, H, KV, hd, window, scale, slopes, nslices, token_list,
                            token_list ? n_listed : n, stream);
   }
   KLLM_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
@@ -430,12 +431,12 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
     if (int rc = nslices == 1                                                                     \
                      ? launch_decode<HDT, decode_waves_whole(HDT)>(                               \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, scale, head_tiles,   \
-                           token_list)                                                            \
+                           block_table, max_pages, page_size, H, KV, window, scale, slopes,          \
+                           head_tiles, token_list)                                                            \
                      : launch_decode<HDT, kDecodeWavesShared>(                                    \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, scale, head_tiles,   \
-                           token_list))                                                           \
+                           block_table, max_pages, page_size, H, KV, window, scale, slopes,          \
+                           head_tiles, token_list))                                                           \
       return rc;                                                                                  \
     break
   switch (hd / 16) {
@@ -454,10 +455,10 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
 extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
                                 const void* cache, const int* positions, const int* span_of_token,
                                 const int* block_table, int max_pages, int page_size, int n, int H,
-                                int KV, int hd, int window, float scale, int nslices, int dtype,
+                                int KV, int hd, int window, float scale, const float* slopes, int nslices, int dtype,
                                 const int* token_list, int n_listed, hipStream_t stream) {
   return attn_decode_run("attn_decode", q, out, part, part_floats, cache, positions, span_of_token,
-                         block_table, max_pages, page_size, n, H, KV, hd, window, scale, nslices, dtype,
+                         block_table, max_pages, page_size, n, H, KV, hd, window, scale, slopes, nslices, dtype,
                          token_list, n_listed, stream);
 }
 
@@ -525,5 +526,5 @@ extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cac
   // (maximum, sum, output of each token, head and slice) that the second one reads.
   return attn_decode_run("attn_decode_static", q, out, part, (long)KLLM_ATTN_DECODE_STATIC_FLOATS, cache,
                          positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window,
-                         scale, nslices, dtype, token_list, n_listed, stream);
+                         scale, nullptr, nslices, dtype, token_list, n_listed, stream);
 }

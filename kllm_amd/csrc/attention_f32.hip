@@ -61,6 +61,7 @@ struct AttnF32Args {
   int count;                   // decode: tokens; prompt: blocks of 128
   int max_pages, page_size, H, KV, hd, window;
   float scale;
+  const float* slopes;         // per head: a bias that grows with the distance to the key (null: none)
   int nslices, col_blocks;     // decode: slices of the keys, blocks of 32 heads per group
   int wg_merge;                // decode: a workgroup's four slices leave one partial result
 };
@@ -145,6 +146,7 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
   const int my_head = DECODE ? h_base + cc : h_base;
   const int my_pos = DECODE ? pos_base : pos_base + cc;
   const int my_start = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const float my_slope = a.slopes ? a.slopes[my_head] : 0.f;
   const int qmax = DECODE ? pos_base : pos_base + ncol - 1;            // last key any column reads
   const int lowest = window > 0 ? max(0, pos_base - window + 1) : 0;   // first key any column reads
   const int first = lowest / 32 * 32;
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
     for (int i = 0; i < 16; ++i) {
       const int key = kb + 8 * (i / 4) + 4 * g + i % 4;
       const bool ok = key <= my_pos && key >= my_start;
-      s[i] = ok ? s[i] * a.scale : -INFINITY;
+      s[i] = ok ? s[i] * a.scale - my_slope * (float)(my_pos - key) : -INFINITY;
       tmax = fmaxf(tmax, s[i]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
@@ -425,7 +427,7 @@ int attn_f32_slices(int n, int KV, int H, int max_keys) {
 
 int attn_f32_decode(const float* q, float* out, float* part, const float* cache, const int* positions,
                     const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                    int H, int KV, int hd, int window, float scale, int nslices, const int* token_list,
+                    int H, int KV, int hd, int window, float scale, const float* slopes, int nslices, const int* token_list,
                     int count, hipStream_t stream) {
   KLLM_REQUIRE(attn_f32_fits(hd, page_size),
                "attn_decode float32: head_dim %d must be a multiple of 8 up to 256 and page_size %d a multiple of 4",
@@ -437,7 +439,7 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
   a.positions = positions; a.span_of_token = span_of_token; a.token_list = token_list;
   a.block_table = block_table; a.count = count;
   a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window;
-  a.scale = scale; a.nslices = nslices; a.col_blocks = (H / KV + 31) / 32;
+  a.scale = scale; a.slopes = slopes; a.nslices = nslices; a.col_blocks = (H / KV + 31) / 32;
   a.wg_merge = nslices % kF32Waves == 0;
   const long items = (long)count * KV * a.col_blocks * nslices;
   if (int rc = dispatch_f32<true>(a, items, stream)) return rc;
@@ -451,7 +453,7 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
 
 int attn_f32_prefill(const float* q, float* out, const float* cache, const int* query_tiles, int n_tiles,
                      const int* span_start, const int* span_pos, const int* block_table, int max_pages,
-                     int page_size, int H, int KV, int hd, int window, float scale, hipStream_t stream) {
+                     int page_size, int H, int KV, int hd, int window, float scale, const float* slopes, hipStream_t stream) {
   KLLM_REQUIRE(attn_f32_fits(hd, page_size),
                "attn_prefill float32: head_dim %d must be a multiple of 8 up to 256 and page_size %d a multiple of 4",
                hd, page_size);
@@ -460,7 +462,7 @@ int attn_f32_prefill(const float* q, float* out, const float* cache, const int* 
   a.query_tiles = query_tiles; a.span_start = span_start; a.span_pos = span_pos;
   a.block_table = block_table; a.count = n_tiles;
   a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window;
-  a.scale = scale; a.nslices = 1; a.col_blocks = 1;
+  a.scale = scale; a.slopes = slopes; a.nslices = 1; a.col_blocks = 1;
   const long items = (long)n_tiles * 4 * H;
   if (int rc = dispatch_f32<false>(a, items, stream)) return rc;
   KLLM_CHECK_LAUNCH("attn_prefill float32");

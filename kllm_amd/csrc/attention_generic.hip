@@ -25,7 +25,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int hd,
-    int window, float scale) {
+    int window, float scale, const float* __restrict__ slopes) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kAttnThreads];
   __shared__ float red[16];
@@ -35,6 +35,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
   const int kvh = h / (H / KV);
   const int pos = positions[t];
   const int len = pos + 1;
+  const float slope = slopes ? slopes[h] : 0.f;   // a bias that grows with the distance to the key
   const int start = (window > 0 && len > window) ? len - window : 0;
   const int* table = block_table + (long)span_of_token[t] * max_pages;
   const long block = (long)page_size * hd;
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
       const T* krow = cache + (((long)page * 2 + 0) * KV + kvh) * block + (long)(key % page_size) * hd;
       float dot = 0.f;
       for (int i = 0; i < hd; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
-      s = dot * scale;
+      s = dot * scale - slope * (float)(pos - key);
     }
     const float cmax = block_max(s, red);
     const float m_new = fmaxf(m, cmax);
@@ -104,7 +105,7 @@ using namespace kllm;
 extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                                  const int* span_of_token, const int* block_table, int max_pages,
                                  int page_size, int n, int H, int KV, int hd, int window,
-                                 float scale, int dtype, hipStream_t stream) {
+                                 float scale, const float* slopes, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table,
                "attn_generic: null pointer");
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_generic: bad heads n=%d H=%d KV=%d", n,
@@ -120,11 +121,11 @@ extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, co
   if (dtype == DT_F32)
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kAttnThreads), 0, stream,
                        (const float*)q, (float*)out, (const float*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, hd, window, scale);
+                       block_table, max_pages, page_size, H, KV, hd, window, scale, slopes);
   else
     hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(kAttnThreads), 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions,
-                       span_of_token, block_table, max_pages, page_size, H, KV, hd, window, scale);
+                       span_of_token, block_table, max_pages, page_size, H, KV, hd, window, scale, slopes);
   KLLM_CHECK_LAUNCH("attn_generic");
   return 0;
 }

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, unsigned page_magic, int H, int KV, int window, float scale, float* __restrict__ part) {
+    int page_size, unsigned page_magic, int H, int KV, int window, float scale, const float* __restrict__ slopes, float* __restrict__ part) {
   typedef PrefillShape<HDT> S;
   constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
@@ -117,6 +117,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const long block = (long)page_size * hd;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const float c2 = scale * 1.4426950408889634f;             // scale * log2(e)
+  // a bias that grows with the distance to the key, in units of raw scores (0: none)
+  const float sb = slopes ? slopes[h] / scale : 0.f;
 
   bf16x8 qb[KS];
 #pragma unroll
@@ -260,6 +262,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(&buf[(32 * b + c) * KLD + 16 * kk + 8 * g]);
         s[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qb[kk], kk == 0 ? zero16 : s[b], 0, 0, 0);
       }
+    if (sb != 0.f) {                                           // the same in every lane
+      const float base = sb * (float)(kb + 4 * g - qpos);
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[b][i] += fmaf(sb, (float)(32 * b + 8 * (i / 4) + i % 4), base);
+    }
     if constexpr (decltype(masked)::value) {
       const int hi = min(qpos, kv_len - 1) - kb - 4 * g, lo = my_start - kb - 4 * g;   // offsets in the tile this lane's query reads
 #pragma unroll
@@ -474,7 +483,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, int H, int KV, int window, float scale) {
+    int page_size, int H, int KV, int window, float scale, const float* __restrict__ slopes) {
   constexpr int hd = 32 * HDT;
   constexpr int KS = hd / 16;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -503,6 +512,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
   const long block = (long)page_size * hd;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const float c2 = scale * 1.4426950408889634f;             // scale * log2(e)
+  // a bias that grows with the distance to the key, in units of raw scores (0: none)
+  const float sb = slopes ? slopes[h] / scale : 0.f;
 
   bf16x8 qb[KS];
 #pragma unroll
@@ -591,6 +602,11 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.k[kk], qb[kk], kk == 0 ? zero16 : s, 0, 0, 0);
     // ---- mask (only where a tile touches an edge), maximum, probabilities.
     // exp(x) is taken as exp2(x * log2 e) with the hardware's exp2.
+    if (sb != 0.f) {                                           // the same in every lane
+      const float base = sb * (float)(kb + 4 * g - qpos);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] += fmaf(sb, (float)(8 * (i / 4) + i % 4), base);
+    }
     const bool inner = kb >= my_start && kb + 31 <= qpos && kb + 32 <= kv_len;   // no mask needed
     if (__any(!inner)) {
       const int hi = min(qpos, kv_len - 1) - kb - 4 * g, lo = my_start - kb - 4 * g;   // offsets in the tile this lane's query reads
@@ -728,7 +744,7 @@ template <int HDT, int PAR>
 static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                                const int* query_tiles, int n_tiles, const int* span_start,
                                const int* span_pos, const int* block_table, int max_pages, int page_size,
-                               int H, int KV, int window, float scale, float* part = nullptr, int nslices = 1) {
+                               int H, int KV, int window, float scale, const float* slopes, float* part = nullptr, int nslices = 1) {
   typedef PrefillShape<HDT> S;
   const size_t lds = (size_t)PAR * 2 * S::kBuf * sizeof(bf16_t);   // also holds the groups' merge
   static int raised = 0;
@@ -740,7 +756,7 @@ static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void
   const unsigned page_magic = (unsigned)(((1UL << 35) + page_size - 1) / page_size);   // ceil(2^35 / page_size)
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid, nslices), dim3(64 * kPrefillWaves * PAR), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale, part);
+                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale, slopes, part);
   if (nslices > 1) {
     const dim3 mgrid(n_tiles * kQueryBlock, ceil_div(H, kMergeWaves));
     hipLaunchKernelGGL((attn_prefill_merge_kernel<(HDT + 1) / 2>), mgrid, dim3(64 * kMergeWaves), 0, stream,
@@ -752,7 +768,7 @@ template <int HDT>
 static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q, void* out, const void* cache,
                                  const int* query_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int window, float scale) {
+                                 int window, float scale, const float* slopes) {
   const size_t lds = (size_t)(kPrefillWaves - 1) * (HDT * 16 + 2) * kWave * sizeof(float);
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
@@ -763,7 +779,7 @@ static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q,
   const int grid = n_tiles * (kQueryBlock / kQueryTile) * H;
   hipLaunchKernelGGL(attn_prefill_split_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale);
+                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale, slopes);
 }
 
 // Which kernel.  One group of waves with the keys through LDS (three workgroups a CU) when
@@ -787,8 +803,8 @@ template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
-                           int H, int KV, int window, float scale, long keys_total, int keys_longest,
-                           float* part, int nslices) {
+                           int H, int KV, int window, float scale, const float* slopes, long keys_total,
+                           int keys_longest, float* part, int nslices) {
   const int cus = device_cus();
   // (the caller asked kllm_attn_prefill_slices: few blocks of a large head.  The slices' results
   // pass through memory and a second kernel, about 10 us for 512 queries of 32 heads; they pay
@@ -796,7 +812,7 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
   if (nslices > 1 && keys_longest >= kPrefillSliceFromKeys) {
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start,
                                                         span_pos, block_table, max_pages, page_size, H, KV, window,
-                                                        scale, part, nslices);
+                                                        scale, slopes, part, nslices);
     return;
   }
   bool chain_bound = true;
@@ -804,14 +820,14 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
     chain_bound = 5 * (keys_total * H / cus) < 6 * (long)keys_longest;
   if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1 || (grid > cus && !chain_bound))
     launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
-                               block_table, max_pages, page_size, H, KV, window, scale);
+                               block_table, max_pages, page_size, H, KV, window, scale, slopes);
   else if (HDT >= 4 || 4 * grid > 3 * cus)
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
                                                         span_start, span_pos, block_table, max_pages, page_size,
-                                                        H, KV, window, scale);
+                                                        H, KV, window, scale, slopes);
   else
     launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
-                              max_pages, page_size, H, KV, window, scale);
+                              max_pages, page_size, H, KV, window, scale, slopes);
 }
 
 }  // namespace kllm
@@ -837,8 +853,8 @@ extern "C" int kllm_attn_prefill_slices(int n_tiles, int H, int hd) {
 extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                                  int n_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int hd, int window, float scale, long keys_total, int keys_longest, float* part,
-                                 long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream) {
+                                 int hd, int window, float scale, const float* slopes, long keys_total, int keys_longest,
+                                 float* part, long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
   KLLM_REQUIRE(keys_total >= 0 && keys_longest >= 0, "attn_prefill: negative numbers of keys");
@@ -848,7 +864,7 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
   if (dtype == DT_F32) {
     KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
     return attn_f32_prefill((const float*)q, (float*)out, (const float*)cache, query_tiles, n_tiles, span_start,
-                            span_pos, block_table, max_pages, page_size, H, KV, hd, window, scale, stream);
+                            span_pos, block_table, max_pages, page_size, H, KV, hd, window, scale, slopes, stream);
   }
   KLLM_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
                "attn_prefill: head_dim %d is not built (32, 64, 96, 128, 192, 256)", hd);
@@ -870,7 +886,7 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \
-                        block_table, max_pages, page_size, H, KV, window, scale, keys_total,      \
+                        block_table, max_pages, page_size, H, KV, window, scale, slopes, keys_total, \
                         keys_longest, part, nslices);                                             \
     break
   switch (hd / 32) {

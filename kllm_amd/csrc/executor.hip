@@ -32,6 +32,13 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_attn_decode),
     KLLM_CMD_OP(kllm_attn_prefill),
     KLLM_CMD_OP(kllm_sample),
+    KLLM_CMD_OP(kllm_add_sinusoid),
+    KLLM_CMD_OP(kllm_unary_act),
+    KLLM_CMD_OP(kllm_group_norm_add),
+    KLLM_CMD_OP(kllm_qk_norm_append),
+    KLLM_CMD_OP(kllm_delta_prep),
+    KLLM_CMD_OP(kllm_delta_scan),
+    KLLM_CMD_OP(kllm_delta_out),
 };
 constexpr int kNumOps = (int)(sizeof(kOps) / sizeof(kOps[0]));
 

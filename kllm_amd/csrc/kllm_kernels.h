@@ -201,11 +201,14 @@ int kllm_fused_linear_max_parts(void);
 int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, const void* w, int n, int m,
                       int k, int tiles_per_wg, hipStream_t stream);
 
-/* Causal attention of n tokens over the paged cache; any head size up to 256. */
+/* Causal attention of n tokens over the paged cache; any head size up to 256.
+ * `slopes` (here and in the other attention entry points; null: none) holds one number per
+ * head: slopes[h] * (query position - key position) is taken off the scaled score, a bias
+ * that grows with the distance to the key. */
 int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                       const int* span_of_token, const int* block_table, int max_pages,
                       int page_size, int n, int H, int KV, int hd, int window, float scale,
-                      int dtype, hipStream_t stream);
+                      const float* slopes, int dtype, hipStream_t stream);
 
 /* Decode attention on the matrix cores: every token's keys are cut into
  * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 4
@@ -223,8 +226,8 @@ int kllm_attn_f32_fits(int hd, int page_size);
 int kllm_attn_decode(const void* q, void* out, float* part, long part_floats, const void* cache,
                      const int* positions, const int* span_of_token, const int* block_table,
                      int max_pages, int page_size, int n, int H, int KV, int hd, int window,
-                     float scale, int nslices, int dtype, const int* token_list, int n_listed,
-                     hipStream_t stream);
+                     float scale, const float* slopes, int nslices, int dtype, const int* token_list,
+                     int n_listed, hipStream_t stream);
 
 /* kllm_attn_decode without a workspace argument and without any allocation: for callers
  * that cannot allocate device memory (code under HIP graph capture, tight serving loops,
@@ -256,14 +259,66 @@ int kllm_attn_decode_static(const void* q, void* out, const void* cache, const i
 int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                       int n_tiles, const int* span_start, const int* span_pos,
                       const int* block_table, int max_pages, int page_size, int H, int KV, int hd,
-                      int window, float scale, long keys_total, int keys_longest, float* part,
-                      long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream);
+                      int window, float scale, const float* slopes, long keys_total, int keys_longest,
+                      float* part, long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream);
 /* nslices of kllm_attn_prefill: how many workgroups share out the keys of a block and head
  * (1: none; more where few blocks of a large head would leave CUs idle; taken only when
  * keys_longest says that the longest block reads 1,280 keys or more).  With more than one,
  * `part` is room for n_rows (the rows of q) x H x nslices x (hd + 2) floats, and the results
  * are merged by a second kernel of the same call. */
 int kllm_attn_prefill_slices(int n_tiles, int H, int hd);
+
+/* x[t][c] += sin(a) for even c, cos(a) for odd c, a = positions[t] * base^(-2 (c/2) / d), angle in double. */
+int kllm_add_sinusoid(float* x, const int* positions, int n, int d, double base, hipStream_t stream);
+
+/* Activations without a gate (`act` below): the gates' two, and xIELU with the two learned
+ * numbers params[0], params[1] (p, q): for z > 0, softplus(p) z^2 + z/2; otherwise
+ * (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */
+#define KLLM_ACT_XIELU 2
+/* out[n][f] = act(sum over s of in[s][n][f]), rounded to out_dtype. */
+int kllm_unary_act(const float* in, int nsplit, long split_stride, void* out, int out_dtype, int n, int f,
+                   int act, const float* params, hipStream_t stream);
+
+/* The norm of a layer whose sub-layers run side by side.  v = x[src] + mult * (sum of d1's ns1
+ * slices + sum of d2's ns2 slices + bias) (each of d1, d2, bias may be null); x[src] = v when
+ * write_x; when out is not null, out[r] = v / sqrt(mean over the channel's group of v^2 + eps)
+ * * w, the d channels being cut into `groups` equal consecutive groups (1: an RMS norm).
+ * src = rows[r] when rows is given (then write_x must be 0), else r. */
+int kllm_group_norm_add(float* x, const float* d1, int ns1, long st1, const float* d2, int ns2, long st2,
+                        const float* bias, float mult, const float* w, void* out, int out_dtype,
+                        const int* rows, int n, int d, int groups, float eps, int write_x,
+                        hipStream_t stream);
+
+/* Between the query/key product and attention where the values are the keys.  qk holds the
+ * sums [nsplit][n][(H + KV) * hd] (queries first).  Biases are added (null: none); the whole
+ * query row and the whole key row are each divided by their root mean square (eps inside the
+ * root) and multiplied by q_w, k_w (null: no norm); the query is multiplied by
+ * 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not); q_out
+ * [n][H*hd] is written, and into the pages of `cache` (null: no append) go the normalised key
+ * as the key and the key before its norm (bias added) as the value. */
+int kllm_qk_norm_append(const float* qk, int nsplit, long split_stride, const float* q_bias,
+                        const float* k_bias, const float* q_w, const float* k_w, float eps, float temp_coef,
+                        int temp_every, void* q_out, void* cache, const int* positions,
+                        const int* span_of_token, const int* block_table, int max_pages, int page_size,
+                        int n, int H, int KV, int hd, int dtype, hipStream_t stream);
+
+/* A recurrent mixer with a matrix state per head, S_t = diag(w) S - (a u)(u^T S) + k v^T,
+ * o = S^T r, u = k / sqrt(sum k^2 + key_eps).
+ * prep: proj [nsplit][n][5*H*hd + L] holds the sums of the products r | k | v | g | a | w1;
+ *   w = exp(-decay_scale * sigmoid(w2 tanh(w1) + w0)), a = sigmoid(a + a_bias); writes scan_in
+ *   [n][H][6][hd] (r, k, v, w, u, a*u) and gate [n][H*hd] = sigmoid(g).  w2 is [H*hd][L] in w_dtype.
+ * scan: one request after the other through state [slots][H][hd][hd] (float32; zero at
+ *   position 0), o_out [n][H*hd]; hd up to kllm_delta_scan_max_dim().
+ * out: out[n][H*hd] = o / sqrt(mean over the head of o^2 + eps) * weight * gate. */
+int kllm_delta_prep(const float* proj, int nsplit, long split_stride, const float* a_bias, const void* w2,
+                    const float* w0, float decay_scale, float key_eps, float* scan_in, float* gate, int n,
+                    int H, int hd, int L, int w_dtype, hipStream_t stream);
+int kllm_delta_scan_max_dim(void);
+int kllm_delta_scan(const float* scan_in, float* o_out, float* state, const int* slots,
+                    const int* span_start, const int* span_pos, int n_spans, int H, int hd,
+                    hipStream_t stream);
+int kllm_delta_out(const float* o, const float* gate, const float* weight, float eps, void* out, int n, int H,
+                   int hd, int dtype, hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

@@ -1,0 +1,150 @@
+// Per-token steps around the products of layers that are not Llama's: additive sinusoidal
+// positions, an activation without a gate (with learned constants), and the norm of a layer
+// whose sub-layers run side by side: it adds a scaled sum of up to two sub-layers' outputs
+// and a bias to the residual stream and normalises the result in groups of channels.
+// Everything here is computed in 32-bit.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+// x[t][c] += sin(angle) for even c, cos(angle) for odd c, angle = p * base^(-2 (c/2) / d) in double.
+__global__ void add_sinusoid_kernel(float* __restrict__ x, const int* __restrict__ positions, int n, int d,
+                                    double log_base) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)n * d) return;
+  const int t = (int)(idx / d), c = (int)(idx % d);
+  const int i = c / 2;
+  const double angle = (double)positions[t] * exp(-(2.0 * i / (double)d) * log_base);
+  x[idx] += (float)((c & 1) ? cos(angle) : sin(angle));
+}
+
+template <typename TOUT>
+__global__ void unary_act_kernel(const float* __restrict__ in, int nsplit, long split_stride,
+                                 TOUT* __restrict__ out, long count, int act, const float* __restrict__ params) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  float a_pos = 0.f, a_neg = 0.f;
+  if (act == ACT_XIELU) {
+    a_pos = softplus_f32(params[0]);
+    a_neg = softplus_f32(params[1]);
+  }
+  float z = 0.f;
+  for (int s = 0; s < nsplit; ++s) z += in[idx + s * split_stride];
+  out[idx] = from_f32<TOUT>(unary_act(z, act, a_pos, a_neg));
+}
+
+constexpr int kGroupNormThreads = 256;
+
+// One workgroup per row.  v = x[src] + mult * (sum of d1's slices + sum of d2's slices + bias);
+// x[src] = v when write_x; out[r] = v / sqrt(mean over the channel's group of v^2 + eps) * w.
+// A group's sum of squares is taken by one wave over a fixed cut of the group, in a fixed
+// order, so a row's result does not depend on what else the launch holds.
+template <typename TOUT>
+__global__ __launch_bounds__(kGroupNormThreads) void group_norm_add_kernel(
+    float* __restrict__ x, const float* __restrict__ d1, int ns1, long st1, const float* __restrict__ d2, int ns2,
+    long st2, const float* __restrict__ bias, float mult, const float* __restrict__ w, TOUT* __restrict__ out,
+    const int* __restrict__ rows, int d, int groups, int segs, float eps, int write_x) {
+  extern __shared__ float v_lds[];          // [d] the row, then [groups * segs] partial sums
+  float* part = v_lds + d;
+  const long r = blockIdx.x;
+  const long src = rows ? rows[r] : r;
+  float* xr = x + src * d;
+  const int tid = threadIdx.x;
+  const bool adds = d1 || d2 || bias;
+  for (int i = tid; i < d; i += kGroupNormThreads) {
+    float v = xr[i];
+    if (adds) {
+      float s = 0.f;
+      if (d1)
+        for (int k = 0; k < ns1; ++k) s += d1[src * d + i + k * st1];
+      if (d2)
+        for (int k = 0; k < ns2; ++k) s += d2[src * d + i + k * st2];
+      if (bias) s += bias[i];
+      v = fmaf(mult, s, v);
+      if (write_x) xr[i] = v;
+    }
+    v_lds[i] = v;
+  }
+  if (!out) return;
+  __syncthreads();
+  const int lane = tid % kWave, wave = tid / kWave, nwaves = kGroupNormThreads / kWave;
+  const int gsz = d / groups;
+  const int seg_len = (gsz + segs - 1) / segs;
+  for (int u = wave; u < groups * segs; u += nwaves) {
+    const int g = u / segs, sg = u % segs;
+    const int lo = g * gsz + sg * seg_len, hi = min(g * gsz + gsz, lo + seg_len);
+    float ss = 0.f;
+    for (int i = lo + lane; i < hi; i += kWave) ss = fmaf(v_lds[i], v_lds[i], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) part[u] = ss;
+  }
+  __syncthreads();
+  for (int i = tid; i < d; i += kGroupNormThreads) {
+    const int g = i / gsz;
+    float ss = 0.f;
+    for (int sg = 0; sg < segs; ++sg) ss += part[g * segs + sg];
+    const float rstd = 1.f / sqrtf(ss / (float)gsz + eps);
+    out[r * d + i] = from_f32<TOUT>(v_lds[i] * rstd * w[i]);
+  }
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_add_sinusoid(float* x, const int* positions, int n, int d, double base, hipStream_t stream) {
+  KLLM_REQUIRE(x && positions, "add_sinusoid: null pointer");
+  KLLM_REQUIRE(n > 0 && d > 0 && base > 0.0, "add_sinusoid: bad sizes n=%d d=%d base=%g", n, d, base);
+  const long count = (long)n * d;
+  hipLaunchKernelGGL(add_sinusoid_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, stream, x, positions, n, d,
+                     log(base));
+  KLLM_CHECK_LAUNCH("add_sinusoid");
+  return 0;
+}
+
+extern "C" int kllm_unary_act(const float* in, int nsplit, long split_stride, void* out, int out_dtype, int n, int f,
+                              int act, const float* params, hipStream_t stream) {
+  KLLM_REQUIRE(in && out, "unary_act: null pointer");
+  KLLM_REQUIRE(n > 0 && f > 0 && nsplit >= 1, "unary_act: bad sizes n=%d f=%d nsplit=%d", n, f, nsplit);
+  KLLM_REQUIRE(act >= 0 && act < UNARY_ACT_COUNT, "unary_act: unknown activation %d", act);
+  KLLM_REQUIRE(act != ACT_XIELU || params, "unary_act: this activation needs its two constants");
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "unary_act: unknown dtype %d", out_dtype);
+  const long count = (long)n * f;
+  const dim3 grid(ceil_div(count, 256));
+  if (out_dtype == DT_F32)
+    hipLaunchKernelGGL(unary_act_kernel<float>, grid, dim3(256), 0, stream, in, nsplit, split_stride, (float*)out,
+                       count, act, params);
+  else
+    hipLaunchKernelGGL(unary_act_kernel<bf16_t>, grid, dim3(256), 0, stream, in, nsplit, split_stride, (bf16_t*)out,
+                       count, act, params);
+  KLLM_CHECK_LAUNCH("unary_act");
+  return 0;
+}
+
+extern "C" int kllm_group_norm_add(float* x, const float* d1, int ns1, long st1, const float* d2, int ns2, long st2,
+                                   const float* bias, float mult, const float* w, void* out, int out_dtype,
+                                   const int* rows, int n, int d, int groups, float eps, int write_x,
+                                   hipStream_t stream) {
+  KLLM_REQUIRE(x, "group_norm_add: null pointer");
+  KLLM_REQUIRE(n > 0 && d > 0 && groups > 0 && d % groups == 0, "group_norm_add: %d channels in %d groups (n=%d)", d,
+               groups, n);
+  KLLM_REQUIRE(!out || w, "group_norm_add: an output needs the norm's weight");
+  KLLM_REQUIRE(!(rows && write_x), "group_norm_add: chosen rows are read only");
+  KLLM_REQUIRE((!d1 || ns1 >= 1) && (!d2 || ns2 >= 1), "group_norm_add: a sum needs at least one slice");
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "group_norm_add: unknown dtype %d", out_dtype);
+  int segs = 1;
+  while (groups * segs < kGroupNormThreads / kWave && d / groups / (2 * segs) >= kWave) segs *= 2;
+  const size_t lds = ((size_t)d + (size_t)groups * segs) * sizeof(float);
+  KLLM_REQUIRE(lds <= 64 * 1024, "group_norm_add: a row of %d channels in %d groups does not fit into LDS", d, groups);
+  if (out_dtype == DT_F32)
+    hipLaunchKernelGGL(group_norm_add_kernel<float>, dim3(n), dim3(kGroupNormThreads), lds, stream, x, d1, ns1, st1,
+                       d2, ns2, st2, bias, mult, w, (float*)out, rows, d, groups, segs, eps, write_x);
+  else
+    hipLaunchKernelGGL(group_norm_add_kernel<bf16_t>, dim3(n), dim3(kGroupNormThreads), lds, stream, x, d1, ns1, st1,
+                       d2, ns2, st2, bias, mult, w, (bf16_t*)out, rows, d, groups, segs, eps, write_x);
+  KLLM_CHECK_LAUNCH("group_norm_add");
+  return 0;
+}

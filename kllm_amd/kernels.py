@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 class KernelError(RuntimeError):
@@ -112,7 +112,7 @@ def _declare(lib):
         "kllm_command_nargs": [I],
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
-        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
         "kllm_device_cus": [],
@@ -126,9 +126,17 @@ def _declare(lib):
         "kllm_calibrate_read": [P, L, P, P],
         "kllm_calibrate_read_workgroups": [],
         "kllm_calibrate_mfma": [I, I, P, P, P],
-        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, I, P],
-        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, L, I, P, L, I, I, I, P],
+        "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, P, I, P],
+        "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, I, P, L, I, I, I, P],
         "kllm_attn_prefill_slices": [I, I, I],
+        "kllm_add_sinusoid": [P, P, I, I, D, P],
+        "kllm_unary_act": [P, I, L, P, I, I, I, I, P, P],
+        "kllm_group_norm_add": [P, P, I, L, P, I, L, P, F, P, P, I, P, I, I, I, F, I, P],
+        "kllm_qk_norm_append": [P, I, L, P, P, P, P, F, F, I, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "kllm_delta_prep": [P, I, L, P, P, P, F, F, P, P, I, I, I, I, I, P],
+        "kllm_delta_scan_max_dim": [],
+        "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, P],
+        "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -145,8 +153,9 @@ def _declare(lib):
 LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_append", "kllm_silu_mul",
              "kllm_sum_splits", "kllm_gemm", "kllm_gemm_swiglu", "kllm_gemv_plain", "kllm_gemv_swiglu",
              "kllm_gemv_resid", "kllm_gemv_rope_append", "kllm_fused_linear", "kllm_attn_generic",
-             "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample")
-DYNAMIC_ARGS = {"kllm_attn_prefill": (15, 16)}     # arguments that may be a StepValue
+             "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_add_sinusoid", "kllm_unary_act",
+             "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out")
+DYNAMIC_ARGS = {"kllm_attn_prefill": (16, 17)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
 
@@ -990,8 +999,17 @@ def sum_splits(parts, out):
                                      _ptr(out, "sum_splits out"), dtype_code(out.dtype), _stream())
 
 
+def _slopes(slopes, n_heads, who):
+    """Pointer of the per-head slopes of a distance bias (float32 [heads]), or null for none."""
+    if slopes is not None and slopes.numel() != n_heads:
+        raise KernelError(f"{who}: {slopes.numel()} slopes for {n_heads} heads")
+    return _ptr(slopes, who + " slopes", torch.float32, True)
+
+
 def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
-                 n_kv_heads, head_dim, window, scale):
+                 n_kv_heads, head_dim, window, scale, slopes=None):
+    """``slopes`` (here and in the other attention wrappers): float32 [heads] or None; slopes[h]
+    times the distance from the query to the key is taken off head h's scaled scores."""
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
@@ -1004,7 +1022,8 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), dtype_code(q.dtype), _stream())
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), _slopes(slopes, n_heads, "attn_generic"),
+        dtype_code(q.dtype), _stream())
 
 
 GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
@@ -1058,7 +1077,7 @@ def attn_prefill_slices(n_tiles, n_heads, head_dim, dtype=torch.bfloat16) -> int
 
 def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, block_table, page_size,
                  n_heads, n_kv_heads, head_dim, window, scale, keys_total=0, keys_longest=0, part=None,
-                 nslices=None):
+                 nslices=None, slopes=None):
     """query_tiles [n_tiles, 2] int32: (first token row, span) of each block of up to
     PREFILL_QUERY_BLOCK consecutive tokens of one span.  ``keys_total`` and
     ``keys_longest``: how many keys the blocks read, all together and the longest block
@@ -1085,7 +1104,7 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
         _ptr(query_tiles, "attn query_tiles", torch.int32), n_tiles,
         _ptr(span_start, "attn span_start", torch.int32), _ptr(span_pos, "attn span_pos", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale),
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), _slopes(slopes, n_heads, "attn_prefill"),
         keys_total if type(keys_total) is StepValue else int(keys_total),
         keys_longest if type(keys_longest) is StepValue else int(keys_longest),
         _ptr(part, "attn part", torch.float32, True) if nslices > 1 else 0, need, nslices, n,
@@ -1093,7 +1112,7 @@ def attn_prefill(q, out, cache, query_tiles, n_tiles, span_start, span_pos, bloc
 
 
 def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page_size, n_heads,
-                n_kv_heads, head_dim, window, scale, nslices, token_list=None, n_listed=0):
+                n_kv_heads, head_dim, window, scale, nslices, token_list=None, n_listed=0, slopes=None):
     n = q.shape[0]
     if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
@@ -1106,7 +1125,8 @@ def attn_decode(q, out, part, cache, positions, span_of_token, block_table, page
         part.numel(), _ptr(cache, "attn cache"), _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), int(nslices), dtype_code(q.dtype),
+        n_heads, n_kv_heads, head_dim, int(window), float(scale), _slopes(slopes, n_heads, "attn_decode"),
+        int(nslices), dtype_code(q.dtype),
         _ptr(token_list, "attn token_list", torch.int32, True), int(n_listed), _stream())
 
 
@@ -1117,3 +1137,152 @@ def sample(out, logits, temperature=None, uniform=None):
     _launch("kllm_sample", "sample", _ptr(out, "sample out", torch.int32), _ptr(logits, "sample logits", torch.float32),
         _ptr(temperature, "sample temperature", torch.float32, True),
         _ptr(uniform, "sample uniform", torch.float32, True), rows, vocab, _stream())
+
+
+# ----------------------------------------------------------------------------- steps of other layer designs
+
+def add_sinusoid(x, positions, base=10000.0):
+    """x [n, d] float32 += the sinusoidal position vector: channel 2i gets sin, 2i + 1 cos of
+    positions[t] * base^(-2i/d)."""
+    n, d = x.shape
+    if positions.numel() < n:
+        raise KernelError("add_sinusoid: positions are too short")
+    _launch("kllm_add_sinusoid", "add_sinusoid", _ptr(x, "add_sinusoid x", torch.float32),
+            _ptr(positions, "add_sinusoid positions", torch.int32), n, d, float(base), _stream())
+
+
+ACT_XIELU = 2
+UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU)
+
+
+def _splits(t, n, cols, who):
+    """(nsplit, stride) of float32 sums [nsplit, n, cols] or [n, cols]."""
+    if t.dtype != torch.float32 or t.shape[-1] != cols or t.shape[-2] != n or t.dim() not in (2, 3):
+        raise KernelError(f"{who}: sums {tuple(t.shape)} {t.dtype} do not fit {n} x {cols} float32")
+    return (t.shape[0], n * cols) if t.dim() == 3 else (1, 0)
+
+
+def unary_act(sums, out, act, params=None):
+    """out [n, f] = act(sums summed over their slices); ``params``: float32 [2], the learned
+    constants of an activation that has them."""
+    n, f = out.shape
+    nsplit, stride = _splits(sums, n, f, "unary_act")
+    if act == ACT_XIELU and (params is None or params.numel() != 2):
+        raise KernelError("unary_act: xielu needs its two constants")
+    _launch("kllm_unary_act", "unary_act", _ptr(sums, "unary_act in", torch.float32), nsplit, stride,
+            _ptr(out, "unary_act out"), dtype_code(out.dtype), n, f, int(act),
+            _ptr(params, "unary_act params", torch.float32, True), _stream())
+
+
+def group_norm_add(x, deltas=(), bias=None, mult=1.0, weight=None, out=None, rows=None, groups=1, eps=0.0,
+                   write_x=None):
+    """x [N, d] float32; v = x + mult * (the deltas' slices summed + bias), written back to x
+    (unless ``rows`` selects rows to read); out [n, d] = v normalised in ``groups`` groups of
+    channels, times weight.  ``deltas``: up to two float32 tensors [N, d] or [nsplit, N, d]."""
+    N, d = x.shape
+    deltas = [t for t in deltas if t is not None]
+    if len(deltas) > 2:
+        raise KernelError("group_norm_add: at most two sums")
+    n = rows.numel() if rows is not None else N
+    if write_x is None:
+        write_x = rows is None and (bool(deltas) or bias is not None)
+    if out is not None and (tuple(out.shape) != (n, d) or weight is None or weight.numel() != d):
+        raise KernelError("group_norm_add: output or weight shape does not fit")
+    if bias is not None and bias.numel() != d:
+        raise KernelError("group_norm_add: bias does not fit")
+    args = []
+    for t in deltas + [None] * (2 - len(deltas)):
+        if t is None:
+            args += [0, 0, 0]
+        else:
+            ns, st = _splits(t, N, d, "group_norm_add")
+            args += [_ptr(t, "group_norm_add delta", torch.float32), ns, st]
+    _launch("kllm_group_norm_add", "group_norm_add", _ptr(x, "group_norm_add x", torch.float32), *args,
+            _ptr(bias, "group_norm_add bias", torch.float32, True), float(mult),
+            _ptr(weight, "group_norm_add weight", torch.float32, True), _ptr(out, "group_norm_add out", None, True),
+            dtype_code(out.dtype) if out is not None else DT_F32, _ptr(rows, "group_norm_add rows", torch.int32, True),
+            n, d, int(groups), float(eps), int(bool(write_x)), _stream())
+
+
+def qk_norm_append(qk, q_out, cache, positions, span_of_token, block_table, page_size, n_heads, n_kv_heads,
+                   head_dim, q_bias=None, k_bias=None, q_weight=None, k_weight=None, eps=0.0, temp_coef=0.0,
+                   temp_every=0):
+    """qk: float32 sums [nsplit, n, (H + KV) * hd] of the query and key products.  Adds the
+    biases, normalises the whole query row and the whole key row (RMS, times their weights),
+    scales the query by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1), writes q_out and
+    appends to the pages: the normalised key as the key, the key before its norm as the value."""
+    n = q_out.shape[0]
+    qd, kd = n_heads * head_dim, n_kv_heads * head_dim
+    nsplit, stride = _splits(qk, n, qd + kd, "qk_norm_append")
+    if q_out.shape[1] != qd:
+        raise KernelError("qk_norm_append: q_out does not fit")
+    for t, size in ((q_bias, qd), (k_bias, kd), (q_weight, qd), (k_weight, kd)):
+        if t is not None and t.numel() != size:
+            raise KernelError("qk_norm_append: a bias or norm weight does not fit")
+    max_pages = 0
+    if cache is not None:
+        if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim) or cache.dtype != q_out.dtype:
+            raise KernelError(f"qk_norm_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
+        max_pages = block_table.shape[1]
+        if span_of_token.numel() < n:
+            raise KernelError("qk_norm_append: index arrays are too short")
+    if positions.numel() < n:
+        raise KernelError("qk_norm_append: index arrays are too short")
+    F32 = torch.float32
+    _launch("kllm_qk_norm_append", "qk_norm_append", _ptr(qk, "qk_norm_append qk", F32), nsplit, stride,
+            _ptr(q_bias, "qk_norm_append q bias", F32, True), _ptr(k_bias, "qk_norm_append k bias", F32, True),
+            _ptr(q_weight, "qk_norm_append q weight", F32, True), _ptr(k_weight, "qk_norm_append k weight", F32, True),
+            float(eps), float(temp_coef), int(temp_every), _ptr(q_out, "qk_norm_append q_out"),
+            _ptr(cache, "qk_norm_append cache", None, True), _ptr(positions, "qk_norm_append positions", torch.int32),
+            _ptr(span_of_token, "qk_norm_append span_of_token", torch.int32, True),
+            _ptr(block_table, "qk_norm_append block_table", torch.int32, True), max_pages, page_size, n,
+            n_heads, n_kv_heads, head_dim, dtype_code(q_out.dtype), _stream())
+
+
+DELTA_SCAN_FIELDS = 6      # per token and head the recurrence reads r, k, v, w, u, a*u
+
+
+def delta_scan_max_dim() -> int:
+    return limit("delta_scan_max_dim")
+
+
+def delta_prep(proj, a_bias, w2, w0, decay_scale, key_eps, scan_in, gate, heads, head_dim):
+    """proj: float32 sums [nsplit, n, 5*H*hd + L] of the products r | k | v | g | a | w1; writes
+    what the recurrence reads, scan_in [n, H, 6, hd], and gate [n, H*hd] = sigmoid(g)."""
+    n, HD = gate.shape
+    L = w2.shape[1]
+    nsplit, stride = _splits(proj, n, 5 * HD + L, "delta_prep")
+    if (HD != heads * head_dim or tuple(scan_in.shape) != (n, heads, DELTA_SCAN_FIELDS, head_dim)
+            or w2.shape[0] != HD or a_bias.numel() != HD or w0.numel() != HD):
+        raise KernelError("delta_prep: shapes do not fit")
+    F32 = torch.float32
+    _launch("kllm_delta_prep", "delta_prep", _ptr(proj, "delta_prep proj", F32), nsplit, stride,
+            _ptr(a_bias, "delta_prep a bias", F32), _ptr(w2, "delta_prep w2"), _ptr(w0, "delta_prep w0", F32),
+            float(decay_scale), float(key_eps), _ptr(scan_in, "delta_prep scan_in", F32),
+            _ptr(gate, "delta_prep gate", F32), n, heads, head_dim, L, dtype_code(w2.dtype), _stream())
+
+
+def delta_scan(scan_in, o_out, state, slots, span_start, span_pos, n_spans):
+    """The recurrence, one request after the other: scan_in [n, H, 6, hd], o_out [n, H*hd], state
+    [slots, H, hd, hd] float32 (started from zero where a span's position is 0)."""
+    n, H, _, hd = scan_in.shape
+    if (tuple(o_out.shape) != (n, H * hd) or tuple(state.shape[1:]) != (H, hd, hd) or state.dtype != torch.float32
+            or slots.numel() < n_spans or span_start.numel() < n_spans + 1 or span_pos.numel() < n_spans):
+        raise KernelError("delta_scan: shapes do not fit")
+    F32, I32 = torch.float32, torch.int32
+    _launch("kllm_delta_scan", "delta_scan", _ptr(scan_in, "delta_scan in", F32), _ptr(o_out, "delta_scan out", F32),
+            _ptr(state, "delta_scan state", F32), _ptr(slots, "delta_scan slots", I32),
+            _ptr(span_start, "delta_scan span_start", I32), _ptr(span_pos, "delta_scan span_pos", I32),
+            int(n_spans), H, hd, _stream())
+
+
+def delta_out(o, gate, weight, eps, out, heads, head_dim):
+    """out [n, H*hd] = each head of o divided by its root mean square, times weight, times gate."""
+    n = o.shape[0]
+    if (tuple(o.shape) != (n, heads * head_dim) or tuple(gate.shape) != tuple(o.shape)
+            or tuple(out.shape) != tuple(o.shape) or weight.numel() != heads * head_dim):
+        raise KernelError("delta_out: shapes do not fit")
+    F32 = torch.float32
+    _launch("kllm_delta_out", "delta_out", _ptr(o, "delta_out o", F32), _ptr(gate, "delta_out gate", F32),
+            _ptr(weight, "delta_out weight", F32), float(eps), _ptr(out, "delta_out out"), n, heads, head_dim,
+            dtype_code(out.dtype), _stream())

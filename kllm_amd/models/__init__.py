@@ -1,3 +1,4 @@
 from . import llama  # registers "LlamaForCausalLM"
+from . import nusilix  # registers "Nusilix"
 
-__all__ = ["llama"]
+__all__ = ["llama", "nusilix"]

@@ -8,7 +8,10 @@ softmax in 32-bit, values, output projection
 
 Parameters: ``hidden``, ``heads``, ``kv_heads``, ``head_dim``, ``window``
 (0: all keys), ``position`` (a PartSpec or None), ``own_kv`` (False: the run
-reads keys and values that another run cached and has no k/v projections).
+reads keys and values that another run cached and has no k/v projections),
+``scale`` (default 1/sqrt(head_dim)), ``distance_slope_bits`` (None: no bias; b:
+head h's scaled scores lose 2^(-b (h+1) / heads) times the distance from the
+query to the key).
 Tensors: ``<prefix>.{q,k,v,o}_proj.weight``.  The three input projections are
 kept as one matrix so that a step reads one weight for them.
 """
@@ -88,7 +91,11 @@ class CausalSelfAttention(Part):
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
             raise ValueError(f"attention: rotary dimension {self.rotary_dim} of a head of {self.head_dim}")
         self.plain_rotation = self.rotary_dim == self.head_dim and not self.interleaved
-        self.scale = 1.0 / math.sqrt(self.head_dim)
+        scale = self.param("scale", None)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        bits = self.param("distance_slope_bits", None)
+        self.slope_bits = float(bits) if bits is not None else None
+        self.slopes = None          # float32 [heads] on the device once bound
         self.q_dim = self.heads * self.head_dim
         self.kv_dim = self.kv_heads * self.head_dim
         self.w_in = None
@@ -103,7 +110,13 @@ class CausalSelfAttention(Part):
         specs.append(WeightSpec(self.tensor_name("o_proj.weight"), (self.hidden, self.q_dim)))
         return specs
 
+    def _bind_slopes(self):
+        if self.slope_bits is not None:
+            values = [2.0 ** (-self.slope_bits * (h + 1) / self.heads) for h in range(self.heads)]
+            self.slopes = torch.tensor(values, dtype=torch.float32, device=self.runtime.device)
+
     def bind(self, weights):
+        self._bind_slopes()
         names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.own_kv else [])
         mats = [weights[self.tensor_name(n)] for n in names]
         self.w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
@@ -202,7 +215,7 @@ class CausalSelfAttention(Part):
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                           self.scale)
+                           self.scale, slopes=self.slopes)
             return
         n = q.shape[0]
         short = ctx.lists.get("attention.spans.short")
@@ -224,7 +237,7 @@ class CausalSelfAttention(Part):
             K.attn_prefill(q, out, cache.pages, blocks, n_blocks, ctx.span_start,
                            ctx.span_pos, cache.block_table, cache.page_size, self.heads,
                            self.kv_heads, self.head_dim, self.window, self.scale, total, longest, part=part,
-                           nslices=slices)
+                           nslices=slices, slopes=self.slopes)
 
     def _keys_read(self, ctx):
         """The step's key counts (see ``step_values``), as the engine worked them out for this
@@ -251,4 +264,71 @@ class CausalSelfAttention(Part):
         part = ctx.buf("attn.part", (n * self.heads * nslices * (self.head_dim + 2),), torch.float32)
         K.attn_decode(q, out, part, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                       cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                      self.scale, nslices, token_list, count)
+                      self.scale, nslices, token_list, count, slopes=self.slopes)
+
+
+@register_part("mixer", "attention_keys_as_values")
+class KeysAsValuesAttention(CausalSelfAttention):
+    """Attention whose values are its keys: there is no value projection, the key as projected
+    is cached as the value and its normalised form as the key.  Queries and keys have biases
+    and are each normalised over the whole projection, all heads at once (RMS, plain weights);
+    the query is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) at position p; no
+    rotation.  Scores, the distance bias, the softmax and the kernels are the base class's.
+
+    Parameters beyond the base class's: ``eps`` (of the two norms), ``q_temp`` (None or a
+    (coef, every) pair), ``bias`` (default True: q, k and the output projection have one).
+    Tensors: ``<prefix>.{q,k,o}.weight``, ``.{q,k,o}.bias``, ``.{q,k}.norm``."""
+    takes_normed = False
+    fills_sink = False
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        if not self.own_kv or self.position is not None:
+            raise ValueError("attention_keys_as_values: keeps its own keys and takes no position part")
+        self.eps = float(self.param("eps"))
+        temp = self.param("q_temp", None)
+        self.temp_coef, self.temp_every = (float(temp[0]), int(temp[1])) if temp else (0.0, 0)
+        if temp and self.temp_every < 1:
+            raise ValueError(f"attention_keys_as_values: q_temp every {self.temp_every} must be positive")
+        self.has_bias = bool(self.param("bias", True))
+        self.q_bias = self.k_bias = self.out_bias = self.q_norm = self.k_norm = None
+
+    def weight_specs(self):
+        specs = [WeightSpec(self.tensor_name("q.weight"), (self.q_dim, self.hidden)),
+                 WeightSpec(self.tensor_name("k.weight"), (self.kv_dim, self.hidden)),
+                 WeightSpec(self.tensor_name("o.weight"), (self.hidden, self.q_dim)),
+                 WeightSpec(self.tensor_name("q.norm"), (self.q_dim,), "vector"),
+                 WeightSpec(self.tensor_name("k.norm"), (self.kv_dim,), "vector")]
+        if self.has_bias:
+            specs += [WeightSpec(self.tensor_name("q.bias"), (self.q_dim,), "vector"),
+                      WeightSpec(self.tensor_name("k.bias"), (self.kv_dim,), "vector"),
+                      WeightSpec(self.tensor_name("o.bias"), (self.hidden,), "vector")]
+        return specs
+
+    def bind(self, weights):
+        self._bind_slopes()
+        self.w_in = torch.cat([weights[self.tensor_name("q.weight")], weights[self.tensor_name("k.weight")]],
+                              dim=0).contiguous()
+        self.w_o = weights[self.tensor_name("o.weight")]
+        self.q_norm = weights[self.tensor_name("q.norm")]
+        self.k_norm = weights[self.tensor_name("k.norm")]
+        if self.has_bias:
+            self.q_bias = weights[self.tensor_name("q.bias")]
+            self.k_bias = weights[self.tensor_name("k.bias")]
+            self.out_bias = weights[self.tensor_name("o.bias")]     # the arrangement adds it with the output
+        self._tiled = {}
+
+    def forward(self, ctx, xn, cache):
+        n = xn.shape[0]
+        dtype = self.runtime.dtype
+        if not cache.write:
+            raise ValueError("attention_keys_as_values: the run writes its own cache")
+        qk = linear(ctx, xn, self.w_in, "attn.qk")
+        q = ctx.buf("attn.q", (n, self.q_dim), dtype)
+        K.qk_norm_append(qk, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
+                         self.heads, self.kv_heads, self.head_dim, q_bias=self.q_bias, k_bias=self.k_bias,
+                         q_weight=self.q_norm, k_weight=self.k_norm, eps=self.eps, temp_coef=self.temp_coef,
+                         temp_every=self.temp_every)
+        out = ctx.buf("attn.out", (n, self.q_dim), dtype)
+        self.attend(ctx, q, out, cache)
+        return linear(ctx, out, self.w_o, "attn.proj")

@@ -213,6 +213,16 @@ class Normed:
 
 
 @dataclass
+class ScaledSum:
+    """What sub-layers that ran side by side leave for the next norm to add to the residual
+    stream: ``mult`` times (the sums of ``deltas``, each float32 [n, d] or [slices, n, d], plus
+    ``bias`` [d]).  A norm that takes one as ``delta`` adds it as it would a plain delta."""
+    deltas: List[torch.Tensor]
+    bias: Optional[torch.Tensor] = None
+    mult: float = 1.0
+
+
+@dataclass
 class StepContext:
     """One step's batch as the parts see it.  All index tensors are int32 on
     the device; the ``h_`` lists are their host copies.

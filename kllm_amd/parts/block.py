@@ -12,7 +12,7 @@ norm's row scale to its own sums (``Normed``).
 
 from __future__ import annotations
 
-from .base import Part, ResidualSink, call_part, make_part, register_part
+from .base import Part, ResidualSink, ScaledSum, call_part, make_part, register_part
 
 
 @register_part("block", "pre_norm")
@@ -84,3 +84,68 @@ class PreNormBlock(Part):
         pending = call_part(self.feed_forward, self.feed_forward.forward, ctx, xn,
                             **self._sink(ctx, x, self.feed_forward, next_norm))
         return x, pending
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Part):
+    """Mixer and feed-forward side by side behind one norm: with h = Norm(x),
+    x' = x + mult * (Mixer(h) + FeedForward(h)).  The layer may have no feed-forward.  Neither
+    output is added by a pass of its own: both travel, with the factor and the bias of a
+    sub-layer's last projection (``out_bias`` of a part, if it has one), as a ``ScaledSum``
+    into the next norm.
+
+    Parameters: ``layer`` (its ``norm_mixer`` is the one norm), ``mult`` (default 1)."""
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        layer = self.param("layer")
+        self.mult = float(self.param("mult", 1.0))
+        self.norm = make_part("norm", layer.norm_mixer, runtime)
+        self.mixer = make_part("mixer", layer.mixer, runtime)
+        self.feed_forward = (make_part("feed_forward", layer.feed_forward, runtime)
+                             if layer.feed_forward is not None else None)
+        self.bias = None
+
+    def parts(self):
+        return [p for p in (self.norm, self.mixer, self.feed_forward) if p is not None]
+
+    def children(self):
+        return self.parts()
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self.parts())
+
+    def weight_specs(self):
+        return [s for p in self.parts() for s in p.weight_specs()]
+
+    def bind(self, weights):
+        for p in self.parts():
+            p.bind(weights)
+        biases = [b for b in (getattr(p, "out_bias", None) for p in self.parts()) if b is not None]
+        self.bias = None
+        if biases:
+            self.bias = biases[0] if len(biases) == 1 else sum(biases[1:], biases[0].clone())
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def read_bytes(self, tokens):
+        out = {}
+        for p in self.parts():
+            out.update(p.read_bytes(tokens))
+        return out
+
+    def flops(self, tokens, keys_read=0.0):
+        return sum(p.flops(tokens, keys_read) for p in self.parts())
+
+    def first_norm(self):
+        return self.norm
+
+    def forward(self, ctx, x, pending, cache):
+        xn = call_part(self.norm, self.norm.forward, ctx, x, delta=pending)
+        deltas = [call_part(self.mixer, self.mixer.forward, ctx, xn, cache)]
+        if self.feed_forward is not None:
+            deltas.append(call_part(self.feed_forward, self.feed_forward.forward, ctx, xn))
+        return x, ScaledSum(deltas, self.bias, self.mult)

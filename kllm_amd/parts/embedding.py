@@ -27,6 +27,9 @@ class TokenEmbedding(Part):
         self.vocab = int(self.param("vocab"))
         self.hidden = int(self.param("hidden"))
         self.table = None
+        # an encoding that acts on the embedded tokens (``on_embedding``): the model calls it
+        pos = self.param("position", None)
+        self.position = runtime.shared_part("position", pos) if pos is not None else None
 
     def weight_specs(self):
         return [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]

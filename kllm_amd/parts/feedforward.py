@@ -95,3 +95,44 @@ class GatedFeedForward(Part):
             if normed is not None:
                 return normed
         return linear(ctx, h, self.w_down, "ffn.down")
+
+
+@register_part("feed_forward", "dense_mlp")
+class DenseFeedForward(Part):
+    """Feed-forward without a gate: down(act(up(x))), no biases.
+
+    Parameters: ``hidden``, ``intermediate``, ``activation`` (one of
+    ``kernels.UNARY_ACTIVATIONS``; "xielu" has two learned constants, the tensor
+    ``<prefix>.act`` [2]).  Tensors: ``<prefix>.{up,down}.weight``."""
+    graph_safe = True
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden = int(self.param("hidden"))
+        self.intermediate = int(self.param("intermediate"))
+        act = self.param("activation", "gelu_tanh")
+        if act not in K.UNARY_ACTIVATIONS:
+            raise ValueError(f"dense_mlp: activation {act!r} is not built (one of {sorted(K.UNARY_ACTIVATIONS)})")
+        self.act = K.UNARY_ACTIVATIONS[act]
+        self.learned = self.act == K.ACT_XIELU
+        self.w_up = self.w_down = self.act_params = None
+
+    def weight_specs(self):
+        specs = [WeightSpec(self.tensor_name("up.weight"), (self.intermediate, self.hidden)),
+                 WeightSpec(self.tensor_name("down.weight"), (self.hidden, self.intermediate))]
+        if self.learned:
+            specs.append(WeightSpec(self.tensor_name("act"), (2,), "vector"))
+        return specs
+
+    def bind(self, weights):
+        self.w_up = weights[self.tensor_name("up.weight")]
+        self.w_down = weights[self.tensor_name("down.weight")]
+        self.act_params = weights[self.tensor_name("act")] if self.learned else None
+
+    def forward(self, ctx, xn):
+        n = xn.shape[0]
+        up = linear(ctx, xn, self.w_up, "ffn.up")
+        h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
+        K.unary_act(up, h, self.act, self.act_params)
+        return linear(ctx, h, self.w_down, "ffn.down")

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from .. import kernels as K
-from .base import Normed, Part, register_part
+from .base import Normed, Part, ScaledSum, register_part
 from .spec import WeightSpec
 
 
@@ -54,4 +54,53 @@ class RMSNorm(Part):
     def add(self, ctx, x, delta):
         if not isinstance(delta, Normed):        # a Normed's sum is in x already
             K.add_rmsnorm(x, delta=delta, write_x=True)
+        return x
+
+
+@register_part("norm", "group_rmsnorm")
+class GroupRMSNorm(Part):
+    """RMS norm in groups: the channels are cut into ``groups`` equal consecutive parts, each
+    is divided by its own sqrt(mean(part^2) + eps), and the whole is multiplied by the weight
+    (``groups`` = 1 is the plain RMS norm).  It also adds what is pending to the residual
+    stream: a plain delta, or a ``ScaledSum`` of sub-layers that ran side by side.
+
+    Parameters: ``size``, ``eps``, ``groups``.  Tensor: ``<prefix>.weight`` [size]."""
+    graph_safe = True
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.size = int(self.param("size"))
+        self.eps = float(self.param("eps"))
+        self.groups = int(self.param("groups", 1))
+        if self.groups < 1 or self.size % self.groups:
+            raise ValueError(f"group_rmsnorm: {self.size} channels do not go into {self.groups} equal groups")
+        self.weight = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.tensor_name("weight"), (self.size,), "vector")]
+
+    def bind(self, weights):
+        self.weight = weights[self.tensor_name("weight")]
+
+    @staticmethod
+    def _sum(delta):
+        if delta is None:
+            return {}
+        if isinstance(delta, Normed):
+            raise ValueError("group_rmsnorm: a residual product cannot stand for this norm")
+        if isinstance(delta, ScaledSum):
+            return {"deltas": delta.deltas, "bias": delta.bias, "mult": delta.mult}
+        return {"deltas": [delta]}
+
+    def forward(self, ctx, x, delta=None, rows=None, tag="xn", normed_ok=False):
+        n = rows.numel() if rows is not None else x.shape[0]
+        out = ctx.buf(tag, (n, self.size), self.runtime.dtype)
+        K.group_norm_add(x, weight=self.weight, out=out, rows=rows, groups=self.groups, eps=self.eps,
+                         **self._sum(delta))
+        return out
+
+    def add(self, ctx, x, delta):
+        if delta is not None:
+            K.group_norm_add(x, **self._sum(delta))
         return x

@@ -20,7 +20,9 @@ class WeightSpec:
 
     role "matrix": held in the engine's compute dtype (bfloat16 or float32);
     role "vector": small per-channel parameters, always held in float32;
-    role "table":  integer tables, held as int32."""
+    role "table":  integer tables, held as int32.
+    A size of -1 in ``shape`` is read from the checkpoint (a width that the configuration
+    does not name); random weights need every size."""
     name: str
     shape: Tuple[int, ...]
     role: str = "matrix"
@@ -75,12 +77,13 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
-    """One layer: an arrangement (block kind) of two norms, a mixer and a
-    feed-forward.  Each layer chooses its own parts."""
+    """One layer: an arrangement (block kind) of norms, a mixer and a
+    feed-forward.  Each layer chooses its own parts; an arrangement that has no
+    use for one of them (one norm for both sub-layers, no feed-forward) leaves it None."""
     mixer: PartSpec
-    feed_forward: PartSpec
-    norm_mixer: PartSpec
-    norm_feed_forward: PartSpec
+    feed_forward: Optional[PartSpec] = None
+    norm_mixer: Optional[PartSpec] = None
+    norm_feed_forward: Optional[PartSpec] = None
     block: str = "pre_norm"
     block_params: Dict[str, Any] = field(default_factory=dict)
 

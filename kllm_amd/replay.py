@@ -34,13 +34,14 @@ from .engine import Engine, EngineOptions, StepEntry
 
 class Replayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16,
-                 device: int = 0, options: Optional[EngineOptions] = None):
+                 device: int = 0, options: Optional[EngineOptions] = None, max_requests: int = 4):
         if options is None:
             # The pool holds max_tokens tokens; a request's count is rounded up
-            # to whole pages (and to 64, which whole pages of 16 divide).
+            # to whole pages (and to 64, which whole pages of 16 divide).  A trace
+            # has at most ``max_requests`` requests alive at a time: that many state slots.
             options = EngineOptions(device=device, dtype=dtype, page_size=page_size,
                                     max_tokens=max_tokens, max_model_len=1 << 30,
-                                    max_requests=64)
+                                    max_requests=max_requests)
         self.engine = Engine.from_dir(model_dir, options)
 
     def step(self, entries: Sequence[dict], end: Sequence = ()) -> Optional[np.ndarray]:
@@ -67,10 +68,12 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--device", type=int, default=0)
+    ap.add_argument("--max-requests", type=int, default=4, help="most requests alive at a time (state slots)")
     args = ap.parse_args(argv)
 
     print("trace_run: loading (kernels are compiled at the first call)", file=sys.stderr, flush=True)
-    rep = Replayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size, device=args.device)
+    rep = Replayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size, device=args.device,
+                   max_requests=args.max_requests)
     os.makedirs(args.out, exist_ok=True)
     print("trace_run: ready", file=sys.stderr, flush=True)
     for line in sys.stdin:

@@ -115,7 +115,7 @@ def check_checkpoint(ckpt: Checkpoint, specs: Sequence[WeightSpec], where: str,
         e = ckpt.entries.get(n)
         if e is None:
             continue
-        if tuple(e.shape) != tuple(s.shape):
+        if len(e.shape) != len(s.shape) or any(w not in (-1, f) for f, w in zip(e.shape, s.shape)):   # -1: any size
             wrong_shape.append((n, tuple(e.shape), tuple(s.shape)))
         ok = _INT_FILE_DTYPES if s.role == "table" else _FLOAT_FILE_DTYPES
         if e.dtype not in ok:
