@@ -307,6 +307,64 @@ def other_engine_points(cfg_small: dict, dtype: str, gemm: str = "hip", page_siz
     return pts
 
 
+# ----------------------------------------------------------------------------- Nusilix beside Llama
+
+# Layer sizes that resemble real models' (random weights): width, heads, KV heads, head size,
+# feed-forward width, layers.  Every fourth layer of the Nusilix model is a recurrent one
+# (width / 64 heads of 64); the Llama model beside it has the same sizes in every layer.
+NUSILIX_SIZES = {
+    "1.1b-sizes": dict(width=2048, heads=32, kv_heads=4, head_dim=64, ff=5632, layers=8, vocab=32000),
+    "8b-sizes": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=14336, layers=4, vocab=32000),
+}
+
+
+def nusilix_config(width, heads, kv_heads, head_dim, ff, layers, vocab, delta_every=4, rank=64) -> dict:
+    entries = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff}
+        if delta_every and i % delta_every == delta_every - 1:
+            entries.append({"type": "general_delta", "mixer": {"heads": width // 64, "dim": 64, "rank": rank}, "mlp": mlp})
+        else:
+            entries.append({"type": "attention", "mlp": mlp,
+                            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim,
+                                      "scale": head_dim ** -0.5, "q_temp": {"coef": 0.3, "every": 256}}})
+    return {"architecture": "Nusilix", "vocab": vocab, "width": width, "residual_mult": 0.5,
+            "norm": {"eps": 1e-6, "groups": 2}, "layers": entries}
+
+
+def llama_config(width, heads, kv_heads, head_dim, ff, layers, vocab) -> dict:
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": layers,
+            "hidden_size": width, "num_attention_heads": heads, "num_key_value_heads": kv_heads, "head_dim": head_dim,
+            "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 10000.0, "max_position_embeddings": 4096,
+            "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "hidden_act": "silu"}
+
+
+def measure_design_pair(sizes: dict, dtype: str, batches=(1, 8), context: int = 2048, prompt: int = 2048,
+                        steps: int = 64, delta_every: int = 4) -> dict:
+    """Prefill and decode throughput of a Nusilix model and of a Llama model of the same layer
+    sizes, one after the other on this GPU."""
+    import gc
+    out = {}
+    for name, cfg in (("nusilix", nusilix_config(delta_every=delta_every, **sizes)), ("llama", llama_config(**sizes))):
+        eng = make_engine(cfg, dtype, max_tokens=max(batches) * context + 2 * prompt, max_model_len=context + 64,
+                          max_requests=max(batches))
+        res = {"weights_GB": round(eng.model.weight_bytes() / 1e9, 3)}
+        pms = measure_prefill(eng, prompt)
+        flops = eng.model.step_flops(prompt, prompt * (prompt + 1) / 2.0, 1)
+        res["prefill"] = {"tokens": prompt, "ms": round(pms, 3), "tok_s": round(prompt * 1e3 / pms, 1),
+                          "frac_of_peak": round(flops / (pms * 1e-3) / PEAK_FLOPS[dtype], 4)}
+        for b in batches:
+            ms, ctx = measure_decode(eng, b, context, steps, 16)
+            need = eng.step_read_bytes([int(ctx)] * b)
+            res[f"decode_b{b}"] = {"ms_per_step": round(ms, 4), "tok_s": round(b * 1e3 / ms, 1),
+                                   "frac_of_hbm": round(need / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        out[name] = res
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def make_engine(cfg: dict, dtype: str, max_tokens: int, seed: int = 0, **opts) -> Engine:
     options = EngineOptions(dtype=dtype, max_tokens=max_tokens, max_requests=max(64, opts.pop("max_requests", 64)),
                             **opts)

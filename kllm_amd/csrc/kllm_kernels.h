@@ -275,9 +275,11 @@ int kllm_add_sinusoid(float* x, const int* positions, int n, int d, double base,
  * numbers params[0], params[1] (p, q): for z > 0, softplus(p) z^2 + z/2; otherwise
  * (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */
 #define KLLM_ACT_XIELU 2
-/* out[n][f] = act(sum over s of in[s][n][f]), rounded to out_dtype. */
-int kllm_unary_act(const float* in, int nsplit, long split_stride, void* out, int out_dtype, int n, int f,
-                   int act, const float* params, hipStream_t stream);
+#define KLLM_ACT_TANH 3
+/* out[n][f] = act(sum over s of in[s][n][f]), rounded to out_dtype; a row of `in` begins every
+ * in_row_stride elements (f if the rows follow each other). */
+int kllm_unary_act(const float* in, int nsplit, long split_stride, int in_row_stride, void* out, int out_dtype,
+                   int n, int f, int act, const float* params, hipStream_t stream);
 
 /* The norm of a layer whose sub-layers run side by side.  v = x[src] + mult * (sum of d1's ns1
  * slices + sum of d2's ns2 slices + bias) (each of d1, d2, bias may be null); x[src] = v when
@@ -306,13 +308,15 @@ int kllm_qk_norm_append(const float* qk, int nsplit, long split_stride, const fl
  * o = S^T r, u = k / sqrt(sum k^2 + key_eps).
  * prep: proj [nsplit][n][5*H*hd + L] holds the sums of the products r | k | v | g | a | w1;
  *   w = exp(-decay_scale * sigmoid(w2 tanh(w1) + w0)), a = sigmoid(a + a_bias); writes scan_in
- *   [n][H][6][hd] (r, k, v, w, u, a*u) and gate [n][H*hd] = sigmoid(g).  w2 is [H*hd][L] in w_dtype.
+ *   [n][H][6][hd] (r, k, v, w, u, a*u) and gate [n][H*hd] = sigmoid(g).  w2 is [H*hd][L] in w_dtype;
+ *   with `low` (sums [low_nsplit][n][H*hd] of w2 tanh(w1), made by a matrix kernel) it is not read.
  * scan: one request after the other through state [slots][H][hd][hd] (float32; zero at
  *   position 0), o_out [n][H*hd]; hd up to kllm_delta_scan_max_dim().
  * out: out[n][H*hd] = o / sqrt(mean over the head of o^2 + eps) * weight * gate. */
 int kllm_delta_prep(const float* proj, int nsplit, long split_stride, const float* a_bias, const void* w2,
-                    const float* w0, float decay_scale, float key_eps, float* scan_in, float* gate, int n,
-                    int H, int hd, int L, int w_dtype, hipStream_t stream);
+                    const float* w0, const float* low, int low_nsplit, long low_stride, float decay_scale,
+                    float key_eps, float* scan_in, float* gate, int n, int H, int hd, int L, int w_dtype,
+                    hipStream_t stream);
 int kllm_delta_scan_max_dim(void);
 int kllm_delta_scan(const float* scan_in, float* o_out, float* state, const int* slots,
                     const int* span_start, const int* span_pos, int n_spans, int H, int hd,

@@ -130,10 +130,10 @@ def _declare(lib):
         "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, I, P, L, I, I, I, P],
         "kllm_attn_prefill_slices": [I, I, I],
         "kllm_add_sinusoid": [P, P, I, I, D, P],
-        "kllm_unary_act": [P, I, L, P, I, I, I, I, P, P],
+        "kllm_unary_act": [P, I, L, I, P, I, I, I, I, P, P],
         "kllm_group_norm_add": [P, P, I, L, P, I, L, P, F, P, P, I, P, I, I, I, F, I, P],
         "kllm_qk_norm_append": [P, I, L, P, P, P, P, F, F, I, P, P, P, P, P, I, I, I, I, I, I, I, P],
-        "kllm_delta_prep": [P, I, L, P, P, P, F, F, P, P, I, I, I, I, I, P],
+        "kllm_delta_prep": [P, I, L, P, P, P, P, I, L, F, F, P, P, I, I, I, I, I, P],
         "kllm_delta_scan_max_dim": [],
         "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, P],
         "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
@@ -1151,8 +1151,8 @@ def add_sinusoid(x, positions, base=10000.0):
             _ptr(positions, "add_sinusoid positions", torch.int32), n, d, float(base), _stream())
 
 
-ACT_XIELU = 2
-UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU)
+ACT_XIELU, ACT_TANH = 2, 3
+UNARY_ACTIVATIONS = dict(ACTIVATIONS, xielu=ACT_XIELU, tanh=ACT_TANH)
 
 
 def _splits(t, n, cols, who):
@@ -1162,15 +1162,19 @@ def _splits(t, n, cols, who):
     return (t.shape[0], n * cols) if t.dim() == 3 else (1, 0)
 
 
-def unary_act(sums, out, act, params=None):
+def unary_act(sums, out, act, params=None, first_column=0):
     """out [n, f] = act(sums summed over their slices); ``params``: float32 [2], the learned
-    constants of an activation that has them."""
+    constants of an activation that has them.  With ``first_column`` the f columns from there
+    of wider sums are taken."""
     n, f = out.shape
-    nsplit, stride = _splits(sums, n, f, "unary_act")
+    cols = sums.shape[-1]
+    nsplit, stride = _splits(sums, n, cols, "unary_act")
+    if first_column < 0 or first_column + f > cols or (first_column == 0 and cols != f):
+        raise KernelError(f"unary_act: columns {first_column} .. {first_column + f} of {cols}")
     if act == ACT_XIELU and (params is None or params.numel() != 2):
         raise KernelError("unary_act: xielu needs its two constants")
-    _launch("kllm_unary_act", "unary_act", _ptr(sums, "unary_act in", torch.float32), nsplit, stride,
-            _ptr(out, "unary_act out"), dtype_code(out.dtype), n, f, int(act),
+    _launch("kllm_unary_act", "unary_act", _ptr(sums, "unary_act in", torch.float32) + 4 * int(first_column), nsplit,
+            stride, cols, _ptr(out, "unary_act out"), dtype_code(out.dtype), n, f, int(act),
             _ptr(params, "unary_act params", torch.float32, True), _stream())
 
 
@@ -1246,19 +1250,22 @@ def delta_scan_max_dim() -> int:
     return limit("delta_scan_max_dim")
 
 
-def delta_prep(proj, a_bias, w2, w0, decay_scale, key_eps, scan_in, gate, heads, head_dim):
+def delta_prep(proj, a_bias, w2, w0, decay_scale, key_eps, scan_in, gate, heads, head_dim, low=None):
     """proj: float32 sums [nsplit, n, 5*H*hd + L] of the products r | k | v | g | a | w1; writes
-    what the recurrence reads, scan_in [n, H, 6, hd], and gate [n, H*hd] = sigmoid(g)."""
+    what the recurrence reads, scan_in [n, H, 6, hd], and gate [n, H*hd] = sigmoid(g).  ``low``:
+    float32 sums [slices, n, H*hd] of w2 . tanh(w1 part) where a matrix kernel made them (the
+    kernel then leaves that product alone)."""
     n, HD = gate.shape
     L = w2.shape[1]
     nsplit, stride = _splits(proj, n, 5 * HD + L, "delta_prep")
+    low_ns, low_st = _splits(low, n, HD, "delta_prep low") if low is not None else (0, 0)
     if (HD != heads * head_dim or tuple(scan_in.shape) != (n, heads, DELTA_SCAN_FIELDS, head_dim)
             or w2.shape[0] != HD or a_bias.numel() != HD or w0.numel() != HD):
         raise KernelError("delta_prep: shapes do not fit")
     F32 = torch.float32
     _launch("kllm_delta_prep", "delta_prep", _ptr(proj, "delta_prep proj", F32), nsplit, stride,
             _ptr(a_bias, "delta_prep a bias", F32), _ptr(w2, "delta_prep w2"), _ptr(w0, "delta_prep w0", F32),
-            float(decay_scale), float(key_eps), _ptr(scan_in, "delta_prep scan_in", F32),
+            _ptr(low, "delta_prep low", F32, True), low_ns, low_st, float(decay_scale), float(key_eps), _ptr(scan_in, "delta_prep scan_in", F32),
             _ptr(gate, "delta_prep gate", F32), n, heads, head_dim, L, dtype_code(w2.dtype), _stream())
 
 

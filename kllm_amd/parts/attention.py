@@ -24,7 +24,7 @@ import torch
 
 from .. import kernels as K
 from .base import Normed, Part, register_part
-from .linear import linear, linear_into, tiled_copy
+from .linear import decode_linear, linear, linear_into, tiled_copy
 from .spec import CacheNeed, WeightSpec
 
 
@@ -316,14 +316,16 @@ class KeysAsValuesAttention(CausalSelfAttention):
             self.q_bias = weights[self.tensor_name("q.bias")]
             self.k_bias = weights[self.tensor_name("k.bias")]
             self.out_bias = weights[self.tensor_name("o.bias")]     # the arrangement adds it with the output
-        self._tiled = {}
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
+                       "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
 
     def forward(self, ctx, xn, cache):
         n = xn.shape[0]
         dtype = self.runtime.dtype
         if not cache.write:
             raise ValueError("attention_keys_as_values: the run writes its own cache")
-        qk = linear(ctx, xn, self.w_in, "attn.qk")
+        qk = decode_linear(ctx, xn, self.w_in, "attn.qk", self._tiled.get("in"))
         q = ctx.buf("attn.q", (n, self.q_dim), dtype)
         K.qk_norm_append(qk, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
                          self.heads, self.kv_heads, self.head_dim, q_bias=self.q_bias, k_bias=self.k_bias,
@@ -331,4 +333,4 @@ class KeysAsValuesAttention(CausalSelfAttention):
                          temp_every=self.temp_every)
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
         self.attend(ctx, q, out, cache)
-        return linear(ctx, out, self.w_o, "attn.proj")
+        return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))

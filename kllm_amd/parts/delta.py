@@ -26,7 +26,7 @@ import torch
 
 from .. import kernels as K
 from .base import Part, register_part
-from .linear import linear
+from .linear import decode_linear, linear, tiled_copy
 from .spec import CacheNeed, WeightSpec
 
 
@@ -34,6 +34,10 @@ from .spec import CacheNeed, WeightSpec
 class GeneralDeltaMixer(Part):
     graph_safe = True
     records_launches = True
+    # From this many tokens on the second product of the decay's low-rank path is a matrix
+    # product of its own (tanh rounded to the compute dtype in between, as any activation that
+    # feeds a product); below, the kernel that prepares the recurrence's inputs does it.
+    LOW_RANK_PRODUCT_ROWS = 17
 
     def __init__(self, spec, runtime):
         super().__init__(spec, runtime)
@@ -68,6 +72,9 @@ class GeneralDeltaMixer(Part):
         self.a_bias = weights[self.tensor_name("a.bias")]
         self.w0 = weights[self.tensor_name("w0")]
         self.norm_weight = weights[self.tensor_name("norm")]
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
+                       "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
 
     def cache_need(self):
         return CacheNeed("state", state_shape=(self.heads, self.head_dim, self.head_dim))
@@ -83,13 +90,19 @@ class GeneralDeltaMixer(Part):
     def forward(self, ctx, xn, cache):
         n = xn.shape[0]
         f32 = torch.float32
-        proj = linear(ctx, xn, self.w_in, "delta.proj")
+        proj = decode_linear(ctx, xn, self.w_in, "delta.proj", self._tiled.get("in"))
+        low = None
+        if n >= self.LOW_RANK_PRODUCT_ROWS:
+            rank = self.w2.shape[1]
+            t = ctx.buf("delta.tanh", (n, rank), self.runtime.dtype)
+            K.unary_act(proj, t, K.ACT_TANH, first_column=5 * self.width)
+            low = linear(ctx, t, self.w2, "delta.low")
         scan_in = ctx.buf("delta.scan_in", (n, self.heads, K.DELTA_SCAN_FIELDS, self.head_dim), f32)
         gate = ctx.buf("delta.gate", (n, self.width), f32)
         K.delta_prep(proj, self.a_bias, self.w2, self.w0, self.decay_scale, self.key_eps, scan_in, gate,
-                     self.heads, self.head_dim)
+                     self.heads, self.head_dim, low=low)
         o = ctx.buf("delta.o", (n, self.width), f32)
         K.delta_scan(scan_in, o, cache.state, cache.slots, ctx.span_start, ctx.span_pos, ctx.n_spans)
         out = ctx.buf("delta.out", (n, self.width), self.runtime.dtype)
         K.delta_out(o, gate, self.norm_weight, self.eps, out, self.heads, self.head_dim)
-        return linear(ctx, out, self.w_o, "delta.o_proj")
+        return decode_linear(ctx, out, self.w_o, "delta.o_proj", self._tiled.get("o"))

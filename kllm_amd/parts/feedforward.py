@@ -13,7 +13,7 @@ import torch
 
 from .. import kernels as K
 from .base import Normed, Part, register_part
-from .linear import linear, linear_into, tiled_copy
+from .linear import decode_linear, linear, linear_into, tiled_copy
 from .spec import WeightSpec
 
 
@@ -129,10 +129,13 @@ class DenseFeedForward(Part):
         self.w_up = weights[self.tensor_name("up.weight")]
         self.w_down = weights[self.tensor_name("down.weight")]
         self.act_params = weights[self.tensor_name("act")] if self.learned else None
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"up": tiled_copy(self.runtime, self.w_up, K.LINEAR_PARTS),
+                       "down": tiled_copy(self.runtime, self.w_down, K.LINEAR_PARTS)}
 
     def forward(self, ctx, xn):
         n = xn.shape[0]
-        up = linear(ctx, xn, self.w_up, "ffn.up")
+        up = decode_linear(ctx, xn, self.w_up, "ffn.up", self._tiled.get("up"))
         h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
         K.unary_act(up, h, self.act, self.act_params)
-        return linear(ctx, h, self.w_down, "ffn.down")
+        return decode_linear(ctx, h, self.w_down, "ffn.down", self._tiled.get("down"))

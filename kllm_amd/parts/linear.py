@@ -275,3 +275,12 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True, w_tiled=None):
     y = ctx.buf(tag + ".sum", (n, m), out_dtype)
     K.sum_splits(parts, y)
     return y
+
+
+def decode_linear(ctx, x, w, tag, w_tiled=None):
+    """``linear`` for a consumer that takes float32 sums either whole or in slices: decode
+    batches of 5 to 16 rows run on the decode-batch kernel with all of K in a workgroup (one
+    result, from the tiled copy of w where there is one); everything else as ``linear`` cuts it."""
+    n = x.shape[0]
+    whole = 4 < n <= 16 and x.dtype == torch.bfloat16 and K.fused_linear_fits(n, x.shape[1])
+    return linear(ctx, x, w, tag, split=not whole, w_tiled=w_tiled)
