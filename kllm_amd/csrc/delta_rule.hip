@@ -23,83 +23,119 @@ constexpr int kScanFields = 6;
 
 // proj: [nsplit][n][5*HD + L], columns r | k | v | g | a | w1.
 // scan_in: [n][H][6][hd]; gate: [n][HD] = sigmoid(g).
+// A workgroup takes one token and as many whole heads as its threads hold channels
+// (blockIdx.y), a thread one channel: every load of a thread is independent of the others.
 template <typename TW>
 __global__ __launch_bounds__(kPrepThreads) void delta_prep_kernel(
     const float* __restrict__ proj, int nsplit, long split_stride, const float* __restrict__ a_bias,
     const TW* __restrict__ w2, const float* __restrict__ w0, const float* __restrict__ low, int low_nsplit,
     long low_stride, float decay_scale, float key_eps, float* __restrict__ scan_in, float* __restrict__ gate, int H,
-    int hd, int L) {
-  extern __shared__ float lds[];           // [L] tanh of the low-rank input, [HD] keys, [H] sums of squares
+    int hd, int L, int heads_per_wg) {
+  extern __shared__ float lds[];           // [L] tanh of the low-rank input, [heads_per_wg * hd] squares of the keys
   float* tl = lds;
-  float* ks = lds + L;
-  float* kss = ks + H * hd;
+  float* ksq = lds + L;
   const int t = blockIdx.x, tid = threadIdx.x;
   const int HD = H * hd, cols = 5 * HD + L;
   const float* in = proj + (long)t * cols;
-  auto column = [&](int c) {
-    float v = 0.f;
-    for (int s = 0; s < nsplit; ++s) v += in[c + s * split_stride];
-    return v;
-  };
+  const int h = blockIdx.y * heads_per_wg + tid / hd, e = tid % hd;
+  const bool live = tid < heads_per_wg * hd && h < H;
+  const int c = live ? h * hd + e : 0;
   if (!low)
-    for (int l = tid; l < L; l += kPrepThreads) tl[l] = tanhf(column(5 * HD + l));
-  for (int c = tid; c < HD; c += kPrepThreads) ks[c] = column(HD + c);
+    for (int l = tid; l < L; l += kPrepThreads) {
+      float v = 0.f;
+      for (int s = 0; s < nsplit; ++s) v += in[5 * HD + l + s * split_stride];
+      tl[l] = tanhf(v);
+    }
+  float f[5] = {0.f, 0.f, 0.f, 0.f, 0.f};  // r, k, v, g, a
+  for (int s = 0; s < nsplit; ++s)
+#pragma unroll
+    for (int q = 0; q < 5; ++q) f[q] += in[q * HD + c + s * split_stride];
+  float lr = w0[c];
+  const float ab = a_bias[c];
+  if (low)
+    for (int sl = 0; sl < low_nsplit; ++sl) lr += low[(long)t * HD + c + sl * low_stride];
+  ksq[tid] = live ? f[1] * f[1] : 0.f;
   __syncthreads();
-  const int lane = tid % kWave, wave = tid / kWave;
-  for (int h = wave; h < H; h += kPrepThreads / kWave) {
-    float ss = 0.f;
-    for (int e = lane; e < hd; e += kWave) ss = fmaf(ks[h * hd + e], ks[h * hd + e], ss);
-    ss = wave_sum(ss);
-    if (lane == 0) kss[h] = ss;
-  }
-  __syncthreads();
-  for (int c = tid; c < HD; c += kPrepThreads) {
-    const int h = c / hd, e = c % hd;
-    float lr = w0[c];
-    if (low) {                               // the low-rank path's second product was made by a matrix kernel
-      for (int sl = 0; sl < low_nsplit; ++sl) lr += low[(long)t * HD + c + sl * low_stride];
+  if (!low) {
+    if (L % 8 == 0 && (((uintptr_t)w2) & 15) == 0) {          // the row in 16- or 32-byte loads, all in flight
+      typedef TW row8 __attribute__((ext_vector_type(8)));
+      const row8* w2r = reinterpret_cast<const row8*>(w2 + (long)c * L);
+      float l0 = 0.f, l1 = 0.f;
+#pragma unroll 4
+      for (int l8 = 0; l8 < L / 8; ++l8) {
+        const row8 wv = w2r[l8];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          l0 = fmaf(to_f32(wv[q]), tl[8 * l8 + q], l0);
+          l1 = fmaf(to_f32(wv[4 + q]), tl[8 * l8 + 4 + q], l1);
+        }
+      }
+      lr += l0 + l1;
     } else {
       const TW* w2r = w2 + (long)c * L;
       for (int l = 0; l < L; ++l) lr = fmaf(to_f32(w2r[l]), tl[l], lr);
     }
-    const float w = expf(-decay_scale * sigmoid_f32(lr));
-    const float a = sigmoid_f32(column(4 * HD + c) + a_bias[c]);
-    const float k = ks[c];
-    const float u = k / sqrtf(kss[h] + key_eps);
-    float* o = scan_in + (((long)t * H + h) * kScanFields) * hd + e;
-    o[0 * hd] = column(c);
-    o[1 * hd] = k;
-    o[2 * hd] = column(2 * HD + c);
-    o[3 * hd] = w;
-    o[4 * hd] = u;
-    o[5 * hd] = a * u;
-    gate[(long)t * HD + c] = sigmoid_f32(column(3 * HD + c));
   }
+  float kss = 0.f;                         // the head's sum of squares, in the order of its channels
+  const float* hsq = ksq + (tid / hd) * hd;
+  for (int q = 0; q < hd; ++q) kss += hsq[q];
+  if (!live) return;
+  const float w = expf(-decay_scale * sigmoid_f32(lr));
+  const float a = sigmoid_f32(f[4] + ab);
+  const float u = f[1] / sqrtf(kss + key_eps);
+  float* o = scan_in + (((long)t * H + h) * kScanFields) * hd + e;
+  o[0 * hd] = f[0];
+  o[1 * hd] = f[1];
+  o[2 * hd] = f[2];
+  o[3 * hd] = w;
+  o[4 * hd] = u;
+  o[5 * hd] = a * u;
+  gate[(long)t * HD + c] = sigmoid_f32(f[3]);
 }
 
+// Sum over the PARTS neighbouring lanes that share a column (PARTS a power of two up to 64), every
+// lane getting the sum: within a row of 16 lanes by data-parallel moves (neighbour, other pair,
+// mirrored half row, mirrored row), which cost an instruction each; across the two rows of a
+// group of 32 by a lane exchange.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);   // (every lane has a source: the move folds into the add)
+  return v + __builtin_bit_cast(float, moved);
+}
+
+template <int PARTS>
+__device__ __forceinline__ float parts_sum(float v) {
+  if (PARTS >= 2) v = dpp_add<0xB1>(v);     // quad_perm [1,0,3,2]
+  if (PARTS >= 4) v = dpp_add<0x4E>(v);     // quad_perm [2,3,0,1]
+  if (PARTS >= 8) v = dpp_add<0x141>(v);    // row_half_mirror
+  if (PARTS >= 16) v = dpp_add<0x140>(v);   // row_mirror
+  if (PARTS >= 32) v += __shfl_xor(v, 16, kWave);
+  if (PARTS >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+constexpr int kScanThreads = 256;
+constexpr int kScanStage = 12;            // elements of a block that a thread stages, at most
+
 // The recurrence.  Columns of the state (value channels) do not see each other, so a workgroup
-// takes a block of columns of one (span, head): thread (j, p) holds rows [8p, 8p + 8) of column
-// j, the PARTS threads of a column are neighbouring lanes of one wave.  A token's vectors are
-// the same for every column; they are staged through LDS, kScanBlock(hd) tokens at a time and
+// takes a block of columns of one (span, head): thread (j, p) holds rows [NR p, NR p + NR) of
+// column j, the PARTS threads of a column are neighbouring lanes of one wave.  A token's vectors
+// are the same for every column; they are staged through LDS, a block of tokens at a time and
 // the next block's loads in flight while this block's tokens are worked through, so that the
 // chain from token to token holds arithmetic and LDS reads only.  Rows beyond hd are padding:
 // their vectors are zero in LDS and their state stays zero.
-constexpr int kScanThreads = 256;
-constexpr int kScanRows = 8;
-constexpr int kScanStage = 12;            // elements of a block that a thread stages, at most
-
-__host__ __device__ inline int scan_block_tokens(int hd_pad) { return hd_pad >= 512 ? 1 : 512 / hd_pad; }
-
-template <int PARTS>
+template <int PARTS, int NR>
 __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
     const float* __restrict__ scan_in, float* __restrict__ o_out, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos, int H,
     int hd) {
-  constexpr int NR = kScanRows;
+  static_assert(NR % 4 == 0, "rows in fours");
   constexpr int HP = PARTS * NR;                       // rows with padding
   constexpr int COLS = kScanThreads / PARTS;           // columns of a workgroup
-  constexpr int TB = HP >= 512 ? 1 : 512 / HP;         // tokens of a block
+  constexpr int TB0 = HP >= 512 ? 1 : 512 / HP;
+  constexpr int TB = TB0 < PARTS ? TB0 : PARTS;        // tokens of a block: lane p of a column keeps token p's output
   constexpr int VEC = kScanFields * HP;                // floats of a token in LDS
+  static_assert(kScanStage * kScanThreads >= TB * VEC, "a block is staged whole");
   __shared__ __attribute__((aligned(16))) float tok[2 * TB * VEC];
   const int span = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int j = blockIdx.z * COLS + tid / PARTS, p = tid % PARTS;
@@ -116,69 +152,112 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
   }
   if (HP != hd)
     for (int i = tid; i < 2 * TB * VEC; i += kScanThreads) tok[i] = 0.f;
+  // Where this thread's elements of a block come from and go to: worked out once.
   const int per_tok = kScanFields * hd;                // floats of a token in memory
-  const long tok_stride = (long)H * per_tok;
+  const int tok_stride = H * per_tok;
   const float* base = scan_in + (long)h * per_tok;
-  float pre[kScanStage];
-  auto ask = [&](int first, int count) {               // the block's elements into registers
+  // A block always runs its TB tokens: where the span ends before, the rest are tokens that
+  // change nothing (decay one, everything else zero), so that the block's code has no branch.
+  int from[kScanStage], to[kScanStage], of_tok[kScanStage];
+  float padv[kScanStage];
 #pragma unroll
-    for (int k = 0; k < kScanStage; ++k) {
-      const int idx = tid + k * kScanThreads;
-      const int tt = idx / per_tok, e = idx % per_tok;
-      pre[k] = (tt < count) ? base[(long)(first + tt) * tok_stride + e] : 0.f;
-    }
+  for (int k = 0; k < kScanStage; ++k) {
+    const int idx = tid + k * kScanThreads;
+    const int tt = idx / per_tok, e = idx % per_tok;
+    of_tok[k] = tt < TB ? tt : (1 << 30);              // beyond the block: never staged
+    from[k] = tt * tok_stride + e;
+    to[k] = tt < TB ? tt * VEC + (e / hd) * HP + e % hd : 0;
+    padv[k] = e / hd == 3 ? 1.f : 0.f;
+  }
+  // Blocks on their way from memory wait in three sets of registers that take turns by name: a
+  // block is asked for three blocks ahead of its use, which covers the memory's latency where
+  // one block's arithmetic does not.
+  float set0[kScanStage], set1[kScanStage], set2[kScanStage];
+  auto ask = [&](float (&pre)[kScanStage], int first) {           // the block's elements into registers
+    const int count = min(TB, t1 - first);                         // <= 0: there is no such block
+    const float* src = base + (long)first * tok_stride;
+#pragma unroll
+    for (int k = 0; k < kScanStage; ++k) pre[k] = (of_tok[k] < count) ? src[from[k]] : 0.f;
   };
-  auto put = [&](float* buf, int count) {
+  auto put = [&](const float (&pre)[kScanStage], float* buf, int first) {
+    const int count = min(TB, t1 - first);
 #pragma unroll
-    for (int k = 0; k < kScanStage; ++k) {
-      const int idx = tid + k * kScanThreads;
-      const int tt = idx / per_tok, e = idx % per_tok;
-      if (tt < count) buf[tt * VEC + (e / hd) * HP + e % hd] = pre[k];
-    }
+    for (int k = 0; k < kScanStage; ++k)
+      if (of_tok[k] < TB) buf[to[k]] = of_tok[k] < count ? pre[k] : padv[k];
   };
   __syncthreads();                                     // the padding is zero before anything is staged
-  ask(t0, min(TB, t1 - t0));
-  put(tok, min(TB, t1 - t0));
+  ask(set0, t0);
+  ask(set1, t0 + TB);
+  ask(set2, t0 + 2 * TB);
+  put(set0, tok, t0);
+  ask(set0, t0 + 3 * TB);
   __syncthreads();
-  int which = 0;
-  for (int tb = t0; tb < t1; tb += TB, which ^= 1) {
-    const int count = min(TB, t1 - tb);
-    const int next_count = min(TB, t1 - tb - TB);      // <= 0: this is the last block
-    if (next_count > 0) ask(tb + TB, next_count);
-    const float* buf = tok + which * TB * VEC;
-    for (int tt = 0; tt < count; ++tt, buf += VEC) {
-      const floatx4* r4 = reinterpret_cast<const floatx4*>(buf + row0);
-      const floatx4* k4 = reinterpret_cast<const floatx4*>(buf + HP + row0);
-      const floatx4* w4 = reinterpret_cast<const floatx4*>(buf + 3 * HP + row0);
-      const floatx4* u4 = reinterpret_cast<const floatx4*>(buf + 4 * HP + row0);
-      const floatx4* a4 = reinterpret_cast<const floatx4*>(buf + 5 * HP + row0);
-      const float vj = buf[2 * HP + (col ? j : 0)];
-      float us = 0.f;
+  const long o_step = (long)H * hd;
+  float o_keep = 0.f;                                  // lane p of a column: the output of the block's token p
+  struct TokenVectors {                                // this thread's rows of a token's vectors
+    floatx4 u[NR / 4], w[NR / 4], k[NR / 4], a[NR / 4], r[NR / 4];
+    float vj;
+  };
+  auto fetch = [&](const float* tv) {
+    TokenVectors T;
 #pragma unroll
-      for (int c = 0; c < NR / 4; ++c) {
-        const floatx4 u = u4[c];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) us = fmaf(u[e], s[4 * c + e], us);
-      }
-#pragma unroll
-      for (int off = 1; off < PARTS; off <<= 1) us += __shfl_xor(us, off, kWave);
-      float o = 0.f;
-#pragma unroll
-      for (int c = 0; c < NR / 4; ++c) {
-        const floatx4 w = w4[c], k = k4[c], a = a4[c], r = r4[c];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float sn = fmaf(w[e], s[4 * c + e], fmaf(k[e], vj, -a[e] * us));
-          s[4 * c + e] = sn;
-          o = fmaf(sn, r[e], o);
-        }
-      }
-#pragma unroll
-      for (int off = 1; off < PARTS; off <<= 1) o += __shfl_xor(o, off, kWave);
-      if (col && p == 0) o_out[((long)(tb + tt) * H + h) * hd + j] = o;
+    for (int c = 0; c < NR / 4; ++c) {
+      T.u[c] = *reinterpret_cast<const floatx4*>(tv + 4 * HP + row0 + 4 * c);
+      T.w[c] = *reinterpret_cast<const floatx4*>(tv + 3 * HP + row0 + 4 * c);
+      T.k[c] = *reinterpret_cast<const floatx4*>(tv + HP + row0 + 4 * c);
+      T.a[c] = *reinterpret_cast<const floatx4*>(tv + 5 * HP + row0 + 4 * c);
+      T.r[c] = *reinterpret_cast<const floatx4*>(tv + row0 + 4 * c);
     }
-    if (next_count > 0) put(tok + (which ^ 1) * TB * VEC, next_count);
+    T.vj = tv[2 * HP + (col ? j : 0)];
+    return T;
+  };
+  auto token = [&](int tt, const TokenVectors& T) {
+    float us0 = 0.f, us1 = 0.f;
+#pragma unroll
+    for (int c = 0; c < NR / 4; ++c) {
+      us0 = fmaf(T.u[c][0], s[4 * c], us0);
+      us1 = fmaf(T.u[c][1], s[4 * c + 1], us1);
+      us0 = fmaf(T.u[c][2], s[4 * c + 2], us0);
+      us1 = fmaf(T.u[c][3], s[4 * c + 3], us1);
+    }
+    const float us = parts_sum<PARTS>(us0 + us1);
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int c = 0; c < NR / 4; ++c)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float sn = fmaf(T.w[c][e], s[4 * c + e], fmaf(T.k[c][e], T.vj, -T.a[c][e] * us));
+        s[4 * c + e] = sn;
+        if (e % 2 == 0) o0 = fmaf(sn, T.r[c][e], o0); else o1 = fmaf(sn, T.r[c][e], o1);
+      }
+    const float o_sum = parts_sum<PARTS>(o0 + o1);     // not part of the chain from token to token
+    o_keep = p == tt ? o_sum : o_keep;
+  };
+  // Block `tb` is worked through from its LDS buffer, a token's vectors read while the token
+  // before it is worked on; then the next block goes from its registers into the other buffer
+  // and those registers are asked for the block three further on.
+  auto block = [&](int tb, float (&next)[kScanStage]) {
+    const int count = min(TB, t1 - tb);
+    const int which = ((tb - t0) / TB) & 1;            // the two LDS buffers take turns
+    const float* buf = tok + which * TB * VEC;
+    TokenVectors cur = fetch(buf);
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) {
+      const TokenVectors nxt = fetch(buf + (tt + 1 < TB ? tt + 1 : tt) * VEC);
+      token(tt, cur);
+      cur = nxt;
+    }
+    if (col && p < count) o_out[(long)(tb + p) * o_step + h * hd + j] = o_keep;
+    put(next, tok + (which ^ 1) * TB * VEC, tb + TB);
+    ask(next, tb + 4 * TB);
     __syncthreads();                                   // the next block is staged; this one is done with
+  };
+  for (int tb = t0; tb < t1; tb += 3 * TB) {           // the three sets of registers take turns by name
+    block(tb, set1);
+    if (tb + TB >= t1) break;
+    block(tb + TB, set2);
+    if (tb + 2 * TB >= t1) break;
+    block(tb + 2 * TB, set0);
   }
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
@@ -218,14 +297,20 @@ extern "C" int kllm_delta_prep(const float* proj, int nsplit, long split_stride,
   KLLM_REQUIRE(n > 0 && H > 0 && hd > 0 && L > 0 && nsplit >= 1, "delta_prep: bad sizes n=%d H=%d hd=%d L=%d", n, H, hd,
                L);
   KLLM_REQUIRE(w_dtype == DT_F32 || w_dtype == DT_BF16, "delta_prep: unknown dtype %d", w_dtype);
-  const size_t lds = ((size_t)L + (size_t)H * hd + H) * sizeof(float);
-  KLLM_REQUIRE(lds <= 64 * 1024, "delta_prep: %d channels do not fit into LDS", H * hd);
+  KLLM_REQUIRE(hd <= kPrepThreads, "delta_prep: heads of %d are not built (up to %d)", hd, kPrepThreads);
+  const int heads_per_wg = kPrepThreads / hd < H ? kPrepThreads / hd : H;
+  const size_t lds = ((size_t)L + kPrepThreads) * sizeof(float);
+  KLLM_REQUIRE(lds <= 64 * 1024, "delta_prep: a low-rank width of %d does not fit into LDS", L);
+  const dim3 grid(n, ceil_div(H, heads_per_wg));
+  KLLM_REQUIRE(grid.y <= 65535, "delta_prep: too many heads for the grid");
   if (w_dtype == DT_F32)
-    hipLaunchKernelGGL(delta_prep_kernel<float>, dim3(n), dim3(kPrepThreads), lds, stream, proj, nsplit, split_stride,
-                       a_bias, (const float*)w2, w0, low, low_nsplit, low_stride, decay_scale, key_eps, scan_in, gate, H, hd, L);
+    hipLaunchKernelGGL(delta_prep_kernel<float>, grid, dim3(kPrepThreads), lds, stream, proj, nsplit, split_stride,
+                       a_bias, (const float*)w2, w0, low, low_nsplit, low_stride, decay_scale, key_eps, scan_in, gate,
+                       H, hd, L, heads_per_wg);
   else
-    hipLaunchKernelGGL(delta_prep_kernel<bf16_t>, dim3(n), dim3(kPrepThreads), lds, stream, proj, nsplit, split_stride,
-                       a_bias, (const bf16_t*)w2, w0, low, low_nsplit, low_stride, decay_scale, key_eps, scan_in, gate, H, hd, L);
+    hipLaunchKernelGGL(delta_prep_kernel<bf16_t>, grid, dim3(kPrepThreads), lds, stream, proj, nsplit, split_stride,
+                       a_bias, (const bf16_t*)w2, w0, low, low_nsplit, low_stride, decay_scale, key_eps, scan_in, gate,
+                       H, hd, L, heads_per_wg);
   KLLM_CHECK_LAUNCH("delta_prep");
   return 0;
 }
@@ -238,20 +323,18 @@ extern "C" int kllm_delta_scan(const float* scan_in, float* o_out, float* state,
   KLLM_REQUIRE(scan_in && o_out && state && slots && span_start && span_pos, "delta_scan: null pointer");
   KLLM_REQUIRE(n_spans > 0 && H > 0 && H <= 65535 && hd > 0 && hd <= 256, "delta_scan: bad sizes spans=%d H=%d hd=%d",
                n_spans, H, hd);
-  // rows in eights over the lanes of a column: 8, 16, 32 ... 256 rows with padding
+  // a column's rows in fours over neighbouring lanes: 4, 8, 16 ... 256 rows with padding
   int parts = 1;
-  while (parts * kScanRows < hd) parts *= 2;
+  while (parts * 4 < hd) parts *= 2;
   const int cols = kScanThreads / parts;
   const dim3 grid(n_spans, H, ceil_div(hd, cols));
-#define KLLM_SCAN(PARTS)                                                                                      \
-  case PARTS:                                                                                                 \
-    static_assert(kScanStage * kScanThreads >= (PARTS * kScanRows >= 512 ? 1 : 512 / (PARTS * kScanRows)) *   \
-                                                   kScanFields * PARTS * kScanRows, "a block is staged whole"); \
-    hipLaunchKernelGGL((delta_scan_kernel<PARTS>), grid, dim3(kScanThreads), 0, stream, scan_in, o_out, state, \
-                       slots, span_start, span_pos, H, hd);                                                   \
+#define KLLM_SCAN(PARTS)                                                                                          \
+  case PARTS:                                                                                                     \
+    hipLaunchKernelGGL((delta_scan_kernel<PARTS, 4>), grid, dim3(kScanThreads), 0, stream, scan_in, o_out, state, \
+                       slots, span_start, span_pos, H, hd);                                                       \
     break
   switch (parts) {
-    KLLM_SCAN(1); KLLM_SCAN(2); KLLM_SCAN(4); KLLM_SCAN(8); KLLM_SCAN(16); KLLM_SCAN(32);
+    KLLM_SCAN(1); KLLM_SCAN(2); KLLM_SCAN(4); KLLM_SCAN(8); KLLM_SCAN(16); KLLM_SCAN(32); KLLM_SCAN(64);
     default: KLLM_FAIL(ERR_ARG, "delta_scan: heads of %d are not built", hd);
   }
 #undef KLLM_SCAN

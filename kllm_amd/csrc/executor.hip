@@ -32,6 +32,7 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_attn_decode),
     KLLM_CMD_OP(kllm_attn_prefill),
     KLLM_CMD_OP(kllm_sample),
+    KLLM_CMD_OP(kllm_gemm_act),
     KLLM_CMD_OP(kllm_add_sinusoid),
     KLLM_CMD_OP(kllm_unary_act),
     KLLM_CMD_OP(kllm_group_norm_add),

@@ -177,7 +177,7 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y, int kslice, int act,
-                                                             int xcds) {
+                                                             const float* __restrict__ act_params, int xcds) {
   typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
@@ -342,6 +342,13 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
       }
     return;
   }
+  // One product: the sums as they are, or (act >= 0) through an activation without a gate.
+  const bool has_act = act >= 0;
+  float a_pos = 0.f, a_neg = 0.f;
+  if (has_act && act == ACT_XIELU) {
+    a_pos = softplus_f32(act_params[0]);
+    a_neg = softplus_f32(act_params[1]);
+  }
 #pragma unroll
   for (int i = 0; i < WTM; ++i)
 #pragma unroll
@@ -351,14 +358,15 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        if (r < n) Y[r * m + c] = from_f32<TOUT>(acc[i][j][e]);
+        const float v = acc[i][j][e];
+        if (r < n) Y[r * m + c] = from_f32<TOUT>(has_act ? unary_act(v, act, a_pos, a_neg) : v);
       }
     }
 }
 
 template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
-                            hipStream_t stream) {
+                            hipStream_t stream, const float* act_params = nullptr) {
   constexpr int MBK = MROW / sizeof(T);
   constexpr int BM = 32 * WTM * WR, BN = 32 * WTN * WC;
   const int tx = ceil_div(m, DUAL ? BN / 2 : BN), ty = ceil_div(n, BM);
@@ -374,7 +382,7 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
     raised = 1;
   }
   hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>), grid, dim3(64 * WR * WC), lds, stream,
-                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act, xcds);
+                     (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act, act_params, xcds);
   return 0;
 }
 
@@ -386,7 +394,7 @@ constexpr long kNarrowBelow = 40000000;   // weights (elements) below which a de
 // the chip's number of CUs.
 template <typename T, typename TOUT, bool DUAL>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
-                       hipStream_t stream) {
+                       hipStream_t stream, const float* act_params = nullptr) {
   const int cus = device_cus();
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
   // A decode batch: tiles of 64 rows, half the products and half the loads of X of 128.  In
@@ -401,13 +409,13 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
     if constexpr (!DUAL) {
       if ((long)m * k < kNarrowBelow) {
         if ((long)ceil_div(m, 64) * nsplit <= cus)
-          return launch_mfma_tile<T, TOUT, DUAL, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream);
-        return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 1, 1>(x, w, y, n, m, k, nsplit, act, stream);
+          return launch_mfma_tile<T, TOUT, DUAL, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+        return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
       }
     }
     if (sizeof(T) == 2 && (long)tx * nsplit <= cus)
-      return launch_mfma_tile<T, TOUT, DUAL, 1, 3>(x, w, y, n, m, k, nsplit, act, stream);
-    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream);
+      return launch_mfma_tile<T, TOUT, DUAL, 1, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   }
   // 256 x 256 tiles (eight waves of 128 x 64, one workgroup a CU) fetch a third less again and
   // are 10-27 % faster (2,048 x 28,672 x 4,096: 499 us against 561 us) where their rounds fill
@@ -437,16 +445,16 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
                            5L * mid * n >= 3L * cus * 256 * ceil_div(n, 256);
     const bool mid_fits = 100 * mid >= 85 * mid_rounds * cus || one_round;
     if (mid_fits && (!big_fits || 3 * mid_rounds <= 4 * rounds))
-      return launch_mfma_tile<T, TOUT, DUAL, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);
+      return launch_mfma_tile<T, TOUT, DUAL, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
     if (big_fits)
-      return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream);
+      return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   }
   const long tall = (long)ceil_div(n, 256) * tx * nsplit;
   if (tall >= 2L * cus && 10 * tall >= 9L * ceil_div(tall, (long)cus) * cus)   // two rounds at least, nine tenths full
-    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, act, stream);
+    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
-  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, act, stream);   // one per CU at most
-  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, act, stream);
+  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);   // one per CU at most
+  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -754,9 +762,9 @@ extern "C" int kllm_gemm(const void* x, const void* w, void* y, int n, int m, in
                  "gemm mfma: nsplit %d leaves an empty slice of K=%d", nsplit, k);
     KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w),
                  "gemm mfma: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
-    int rc = f32 ? launch_mfma<float, float, false>(x, w, y, n, m, k, nsplit, 0, stream)
-             : out_dtype == DT_F32 ? launch_mfma<bf16_t, float, false>(x, w, y, n, m, k, nsplit, 0, stream)
-                                   : launch_mfma<bf16_t, bf16_t, false>(x, w, y, n, m, k, 1, 0, stream);
+    int rc = f32 ? launch_mfma<float, float, false>(x, w, y, n, m, k, nsplit, -1, stream)
+             : out_dtype == DT_F32 ? launch_mfma<bf16_t, float, false>(x, w, y, n, m, k, nsplit, -1, stream)
+                                   : launch_mfma<bf16_t, bf16_t, false>(x, w, y, n, m, k, 1, -1, stream);
     if (rc) return rc;
     KLLM_CHECK_LAUNCH("gemm mfma");
     return 0;
@@ -857,5 +865,24 @@ extern "C" int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, i
                                : launch_mfma<bf16_t, bf16_t, true>(x, w_gate_up, h, n, f, k, 1, act, stream))
     return rc;
   KLLM_CHECK_LAUNCH("gemm_swiglu");
+  return 0;
+}
+
+// h[n][m] = act(x . w^T) in dtype, the activation (one without a gate) in the product's epilogue.
+extern "C" int kllm_gemm_act(const void* x, const void* w, void* h, int n, int m, int k, int dtype, int act,
+                             const float* act_params, hipStream_t stream) {
+  KLLM_REQUIRE(x && w && h, "gemm_act: null pointer");
+  KLLM_REQUIRE(act >= 0 && act < UNARY_ACT_COUNT, "gemm_act: unknown activation %d", act);
+  KLLM_REQUIRE(act != ACT_XIELU || act_params, "gemm_act: this activation needs its two constants");
+  KLLM_REQUIRE(n > 0 && m > 0 && k > 0, "gemm_act: bad sizes n=%d m=%d k=%d", n, m, k);
+  KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "gemm_act: unknown dtype %d", dtype);
+  const int chunk = dtype == DT_F32 ? 4 : 8;
+  KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w),
+               "gemm_act: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
+  KLLM_REQUIRE((long)n * m < (1L << 31), "gemm_act: sizes overflow");
+  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, false>(x, w, h, n, m, k, 1, act, stream, act_params)
+                               : launch_mfma<bf16_t, bf16_t, false>(x, w, h, n, m, k, 1, act, stream, act_params))
+    return rc;
+  KLLM_CHECK_LAUNCH("gemm_act");
   return 0;
 }

@@ -101,6 +101,11 @@ int kllm_gemm(const void* x, const void* w, void* y, int n, int m, int k, int dt
 int kllm_gemm_swiglu(const void* x, const void* w_gate_up, void* h, int n, int f, int k, int dtype,
                      int act, hipStream_t stream);
 
+/* h[n][m] = act(x . w^T) on the MFMA tiles, h in dtype; act is one of the activations without
+ * a gate (see kllm_unary_act), act_params its learned constants where it has them. */
+int kllm_gemm_act(const void* x, const void* w, void* h, int n, int m, int k, int dtype, int act,
+                  const float* act_params, hipStream_t stream);
+
 /* Products for up to 8 rows of x with the whole of K in one wave (no partial
  * sums) and the next elementwise step in the epilogue.  m even, K a multiple
  * of 8 (bfloat16) or 4 (float32).

@@ -10,15 +10,20 @@
 
 namespace kllm {
 
-// x[t][c] += sin(angle) for even c, cos(angle) for odd c, angle = p * base^(-2 (c/2) / d) in double.
+// x[t][2i] += sin(angle), x[t][2i + 1] += cos(angle), angle = p * base^(-2i / d) in double; a thread
+// takes one angle.
 __global__ void add_sinusoid_kernel(float* __restrict__ x, const int* __restrict__ positions, int n, int d,
                                     double log_base) {
+  const int pairs = (d + 1) / 2;
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (long)n * d) return;
-  const int t = (int)(idx / d), c = (int)(idx % d);
-  const int i = c / 2;
+  if (idx >= (long)n * pairs) return;
+  const int t = (int)(idx / pairs), i = (int)(idx % pairs);
   const double angle = (double)positions[t] * exp(-(2.0 * i / (double)d) * log_base);
-  x[idx] += (float)((c & 1) ? cos(angle) : sin(angle));
+  double sn, cs;
+  sincos(angle, &sn, &cs);
+  float* row = x + (long)t * d;
+  row[2 * i] += (float)sn;
+  if (2 * i + 1 < d) row[2 * i + 1] += (float)cs;
 }
 
 template <typename TOUT>
@@ -168,7 +173,7 @@ using namespace kllm;
 extern "C" int kllm_add_sinusoid(float* x, const int* positions, int n, int d, double base, hipStream_t stream) {
   KLLM_REQUIRE(x && positions, "add_sinusoid: null pointer");
   KLLM_REQUIRE(n > 0 && d > 0 && base > 0.0, "add_sinusoid: bad sizes n=%d d=%d base=%g", n, d, base);
-  const long count = (long)n * d;
+  const long count = (long)n * ((d + 1) / 2);
   hipLaunchKernelGGL(add_sinusoid_kernel, dim3(ceil_div(count, 256)), dim3(256), 0, stream, x, positions, n, d,
                      log(base));
   KLLM_CHECK_LAUNCH("add_sinusoid");

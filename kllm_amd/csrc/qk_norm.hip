@@ -21,23 +21,48 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
     float temp_coef, int temp_every, T* __restrict__ q_out, T* __restrict__ cache, const int* __restrict__ positions,
     const int* __restrict__ span_of_token, const int* __restrict__ block_table, int max_pages, int page_size, int H,
     int KV, int hd) {
-  extern __shared__ float row[];            // [H*hd + KV*hd]
+  extern __shared__ float row[];            // [H*hd + KV*hd] the sums, then as many norm weights
   __shared__ float red[16];
   const int t = blockIdx.x, tid = threadIdx.x;
   const int qd = H * hd, kd = KV * hd, cols = qd + kd;
   const float* in = qk + (long)t * cols;
+  float* wrow = row + cols;
   float ssq = 0.f, ssk = 0.f;
-  for (int i = tid; i < cols; i += kQkThreads) {
-    float v = 0.f;
-    for (int s = 0; s < nsplit; ++s) v += in[i + s * split_stride];
-    if (i < qd) {
-      if (q_bias) v += q_bias[i];
-      ssq = fmaf(v, v, ssq);
-    } else {
-      if (k_bias) v += k_bias[i - qd];
-      ssk = fmaf(v, v, ssk);
+  // eight of a thread's elements at a time: their loads (every slice, the bias) go out together
+  for (int i0 = tid; i0 < cols; i0 += 8 * kQkThreads) {
+    float v[8], wv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kQkThreads;
+      v[u] = 0.f;
+      wv[u] = 1.f;
+      if (i < cols) {
+        if (i < qd) {
+          if (q_w) wv[u] = q_w[i];
+        } else if (k_w) {
+          wv[u] = k_w[i - qd];
+        }
+        if (i < qd) {
+          if (q_bias) v[u] = q_bias[i];
+        } else if (k_bias) {
+          v[u] = k_bias[i - qd];
+        }
+      }
     }
-    row[i] = v;
+    for (int s = 0; s < nsplit; ++s)
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * kQkThreads;
+        v[u] += i < cols ? in[i + s * split_stride] : 0.f;
+      }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kQkThreads;
+      if (i >= cols) continue;
+      if (i < qd) ssq = fmaf(v[u], v[u], ssq); else ssk = fmaf(v[u], v[u], ssk);
+      row[i] = v[u];
+      wrow[i] = wv[u];
+    }
   }
   ssq = block_sum(ssq, red);
   ssk = block_sum(ssk, red);
@@ -46,9 +71,10 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
   if (temp_every > 0) qmul = 1.f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.f);
   const float rq = q_w ? 1.f / sqrtf(ssq / (float)qd + eps) : 1.f;
   const float rk = k_w ? 1.f / sqrtf(ssk / (float)kd + eps) : 1.f;
+#pragma unroll 4
   for (int i = tid; i < qd; i += kQkThreads) {
     float v = row[i];
-    if (q_w) v = v * rq * q_w[i];
+    if (q_w) v = v * rq * wrow[i];
     q_out[(long)t * qd + i] = from_f32<T>(v * qmul);
   }
   if (!cache) return;
@@ -58,7 +84,7 @@ __global__ __launch_bounds__(kQkThreads) void qk_norm_append_kernel(
   for (int i = tid; i < kd; i += kQkThreads) {
     const int kvh = i / hd, e = i % hd;
     const float raw = row[qd + i];
-    const float key = k_w ? raw * rk * k_w[i] : raw;
+    const float key = k_w ? raw * rk * wrow[qd + i] : raw;
     T* kpage = cache + (((long)page * 2 + 0) * KV + kvh) * block;
     T* vpage = cache + (((long)page * 2 + 1) * KV + kvh) * block;
     kpage[(long)slot * hd + e] = from_f32<T>(key);
@@ -81,7 +107,7 @@ extern "C" int kllm_qk_norm_append(const float* qk, int nsplit, long split_strid
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && hd > 0 && nsplit >= 1, "qk_norm_append: bad sizes n=%d H=%d KV=%d hd=%d", n,
                H, KV, hd);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "qk_norm_append: unknown dtype %d", dtype);
-  const size_t lds = (size_t)(H + KV) * hd * sizeof(float);
+  const size_t lds = 2 * (size_t)(H + KV) * hd * sizeof(float);
   KLLM_REQUIRE(lds <= 64 * 1024, "qk_norm_append: %d query and key channels do not fit into LDS", (H + KV) * hd);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(qk_norm_append_kernel<float>, dim3(n), dim3(kQkThreads), lds, stream, qk, nsplit, split_stride,

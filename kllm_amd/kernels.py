@@ -129,6 +129,7 @@ def _declare(lib):
         "kllm_attn_decode": [P, P, P, L, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, P, I, P],
         "kllm_attn_prefill": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, I, P, L, I, I, I, P],
         "kllm_attn_prefill_slices": [I, I, I],
+        "kllm_gemm_act": [P, P, P, I, I, I, I, I, P, P],
         "kllm_add_sinusoid": [P, P, I, I, D, P],
         "kllm_unary_act": [P, I, L, I, P, I, I, I, I, P, P],
         "kllm_group_norm_add": [P, P, I, L, P, I, L, P, F, P, P, I, P, I, I, I, F, I, P],
@@ -153,7 +154,7 @@ def _declare(lib):
 LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_append", "kllm_silu_mul",
              "kllm_sum_splits", "kllm_gemm", "kllm_gemm_swiglu", "kllm_gemv_plain", "kllm_gemv_swiglu",
              "kllm_gemv_resid", "kllm_gemv_rope_append", "kllm_fused_linear", "kllm_attn_generic",
-             "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_add_sinusoid", "kllm_unary_act",
+             "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_gemm_act", "kllm_add_sinusoid", "kllm_unary_act",
              "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out")
 DYNAMIC_ARGS = {"kllm_attn_prefill": (16, 17)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
@@ -1176,6 +1177,19 @@ def unary_act(sums, out, act, params=None, first_column=0):
     _launch("kllm_unary_act", "unary_act", _ptr(sums, "unary_act in", torch.float32) + 4 * int(first_column), nsplit,
             stride, cols, _ptr(out, "unary_act out"), dtype_code(out.dtype), n, f, int(act),
             _ptr(params, "unary_act params", torch.float32, True), _stream())
+
+
+def gemm_act(x, w, h, act, params=None):
+    """h [n, m] = act(x . w^T) on the MFMA tiles, the activation (one without a gate) in the
+    product's epilogue; h in the dtype of x and w."""
+    n, k = x.shape
+    m = w.shape[0]
+    if w.shape[1] != k or x.dtype != w.dtype or tuple(h.shape) != (n, m) or h.dtype != x.dtype:
+        raise KernelError(f"gemm_act: x {tuple(x.shape)}, w {tuple(w.shape)}, h {tuple(h.shape)} do not fit")
+    if act == ACT_XIELU and (params is None or params.numel() != 2):
+        raise KernelError("gemm_act: xielu needs its two constants")
+    _launch("kllm_gemm_act", "gemm_act", _ptr(x, "gemm_act x"), _ptr(w, "gemm_act w"), _ptr(h, "gemm_act h"), n, m, k,
+            dtype_code(x.dtype), int(act), _ptr(params, "gemm_act params", torch.float32, True), _stream())
 
 
 def group_norm_add(x, deltas=(), bias=None, mult=1.0, weight=None, out=None, rows=None, groups=1, eps=0.0,

@@ -135,7 +135,11 @@ class DenseFeedForward(Part):
 
     def forward(self, ctx, xn):
         n = xn.shape[0]
-        up = decode_linear(ctx, xn, self.w_up, "ffn.up", self._tiled.get("up"))
         h = ctx.buf("ffn.h", (n, self.intermediate), self.runtime.dtype)
-        K.unary_act(up, h, self.act, self.act_params)
+        if (n > 128 and self.runtime.options.get("gemm") != "library" and self.runtime.options.get("gemm_algo") is None
+                and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
+            K.gemm_act(xn, self.w_up, h, self.act, self.act_params)      # prompts: the activation in the product's epilogue
+        else:
+            up = decode_linear(ctx, xn, self.w_up, "ffn.up", self._tiled.get("up"))
+            K.unary_act(up, h, self.act, self.act_params)
         return decode_linear(ctx, h, self.w_down, "ffn.down", self._tiled.get("down"))
