@@ -108,7 +108,12 @@ extern "C" int kllm_qk_norm_append(const float* qk, int nsplit, long split_strid
                H, KV, hd);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "qk_norm_append: unknown dtype %d", dtype);
   const size_t lds = 2 * (size_t)(H + KV) * hd * sizeof(float);
-  KLLM_REQUIRE(lds <= 64 * 1024, "qk_norm_append: %d query and key channels do not fit into LDS", (H + KV) * hd);
+  KLLM_REQUIRE(lds <= 160 * 1024, "qk_norm_append: %d query and key channels do not fit into LDS", (H + KV) * hd);
+  if (lds > 64 * 1024) {
+    const void* fn = dtype == DT_F32 ? (const void*)qk_norm_append_kernel<float> : (const void*)qk_norm_append_kernel<bf16_t>;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) KLLM_FAIL((int)e, "qk_norm_append: cannot raise the LDS limit: %s", hipGetErrorString(e));
+  }
   if (dtype == DT_F32)
     hipLaunchKernelGGL(qk_norm_append_kernel<float>, dim3(n), dim3(kQkThreads), lds, stream, qk, nsplit, split_stride,
                        q_bias, k_bias, q_w, k_w, eps, temp_coef, temp_every, (float*)q_out, (float*)cache, positions,

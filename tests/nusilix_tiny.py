@@ -8,6 +8,9 @@ N2: heads of 64 (the bfloat16 prompt and decode kernels), one KV head, one norm 
 N3: heads of 32 and of 128, as many KV heads as heads on one layer, three norm groups, a width
     that is no power of two, a recurrence with heads of 64 and a low-rank width that is no
     multiple of 8.
+N5: recurrent layers only (no pages at all), heads of 20, a low-rank width of 5.
+N6: attention only (no state slots), as many KV heads as heads, heads of 20 (the kernel for every
+    size in both number formats), an odd vocabulary, a temperature step at every position.
 N4: heads of 24 in both mixers (sizes that only the kernel for every size takes in bfloat16),
     three recurrent heads, two recurrent layers in a row.
 """
@@ -44,6 +47,9 @@ CONFIGS = {
                           attn(4, 1, 64, coef=0.5, every=8, ff=160)], 1e-6, 1, 1.0),
     "N3": _cfg(101, 96, [attn(8, 1, 32, every=16, ff=64), delta(1, 64, rank=12, ff=56),
                          attn(2, 2, 128, coef=0.1, every=3)], 1e-4, 3, 0.7),
+    "N5": _cfg(50, 40, [delta(2, 20, rank=5, ff=24), delta(2, 20, rank=5)], 1e-6, 2, 0.6),
+    "N6": _cfg(61, 48, [attn(5, 5, 20, coef=0.25, every=1, ff=32), attn(5, 5, 20, coef=0.25, every=1, ff=32)],
+               1e-5, 1, 1.0),
     "N4": _cfg(77, 72, [attn(6, 3, 24, every=7, ff=40), delta(3, 24, rank=4), delta(3, 24, rank=4, ff=48)],
                1e-5, 4, 0.35),
 }
