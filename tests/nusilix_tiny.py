@@ -11,6 +11,8 @@ N3: heads of 32 and of 128, as many KV heads as heads on one layer, three norm g
 N5: recurrent layers only (no pages at all), heads of 20, a low-rank width of 5.
 N6: attention only (no state slots), as many KV heads as heads, heads of 20 (the kernel for every
     size in both number formats), an odd vocabulary, a temperature step at every position.
+N7: a width of 50 in five norm groups (no multiple of 4 or 8 anywhere: the plain products and the
+    norm kernel for every size), heads of 8 and 12, a low-rank width of 3, a factor above 1.
 N4: heads of 24 in both mixers (sizes that only the kernel for every size takes in bfloat16),
     three recurrent heads, two recurrent layers in a row.
 """
@@ -50,6 +52,8 @@ CONFIGS = {
     "N5": _cfg(50, 40, [delta(2, 20, rank=5, ff=24), delta(2, 20, rank=5)], 1e-6, 2, 0.6),
     "N6": _cfg(61, 48, [attn(5, 5, 20, coef=0.25, every=1, ff=32), attn(5, 5, 20, coef=0.25, every=1, ff=32)],
                1e-5, 1, 1.0),
+    "N7": _cfg(33, 50, [attn(2, 1, 8, every=4, ff=30), delta(2, 12, rank=3, ff=22), attn(2, 1, 8, every=4)],
+               1e-5, 5, 1.3),
     "N4": _cfg(77, 72, [attn(6, 3, 24, every=7, ff=40), delta(3, 24, rank=4), delta(3, 24, rank=4, ff=48)],
                1e-5, 4, 0.35),
 }

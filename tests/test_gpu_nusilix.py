@@ -26,7 +26,7 @@ DTYPES = ["float32", "bfloat16"]
 TD = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 F64 = torch.float64
 # Logits: root mean square of the difference (mean taken off) over that of the plain model's
-# logits.  Measured over all tests of this file: float32 at most 3.1e-6, bfloat16 at most 1.23e-2.
+# logits.  Measured over all tests of this file: float32 at most 3.1e-6, bfloat16 at most 1.54e-2.
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 WORST = {"float32": 0.0, "bfloat16": 0.0}
 
@@ -316,7 +316,7 @@ def compare(rows, want, dtype, requests):
 
 
 CASES = [("N1", [1, 5, 33, 130]), ("N2", [2, 17, 140]), ("N3", [3, 64, 65, 150]), ("N4", [90, 31]),
-         ("N5", [70, 4]), ("N6", [49, 80])]
+         ("N5", [70, 4]), ("N6", [49, 80]), ("N7", [66, 19, 140])]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
