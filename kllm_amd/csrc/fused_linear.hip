@@ -59,6 +59,9 @@ constexpr int FL_LDS_MAX = 160 * 1024;
 constexpr int FL_TILE = 16 * 17;    // floats of one wave's partial tile in LDS: [x row][w row], padded
 
 enum : int { FL_PARTS = 0, FL_RESID = 1, FL_SWIGLU = 2, FL_ROPE = 3 };
+// FL_PARTS with act >= FL_UNARY: y is bfloat16 [n][m] = unary_act(sums, act - FL_UNARY), the
+// activation's learned constants (if it has any) behind norm_w.
+constexpr int FL_UNARY = 16;
 
 struct FlOut {
   void* y;
@@ -393,7 +396,18 @@ __global__ __launch_bounds__(64 * NW) void fused_linear_kernel(const bf16_t* __r
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) v += pb[(w * NT + t) * FL_TILE + xc * 17 + r16];
-        if (row < m && xr < n) reinterpret_cast<float*>(out.y)[((long)blockIdx.y * n + xr) * m + row] = v;
+        if (row < m && xr < n) {
+          if (out.act >= FL_UNARY) {       // an activation without a gate on the sums, stored in bfloat16
+            float a_pos = 0.f, a_neg = 0.f;
+            if (out.act - FL_UNARY == ACT_XIELU) {
+              a_pos = softplus_f32(out.norm_w[0]);
+              a_neg = softplus_f32(out.norm_w[1]);
+            }
+            reinterpret_cast<bf16_t*>(out.y)[(long)xr * m + row] = (bf16_t)unary_act(v, out.act - FL_UNARY, a_pos, a_neg);
+          } else {
+            reinterpret_cast<float*>(out.y)[((long)blockIdx.y * n + xr) * m + row] = v;
+          }
+        }
       }
     } else if (EP == FL_RESID) {
       if (tid < 256) {
@@ -669,6 +683,14 @@ extern "C" int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOu
   out.act = yout->act;
   out.tiled = yout->tiled ? 1 : 0;
   KLLM_REQUIRE(ep != FL_SWIGLU || (out.act >= 0 && out.act < ACT_COUNT), "fused_linear: unknown activation %d", out.act);
+  if (ep == FL_PARTS && out.act >= FL_UNARY) {
+    KLLM_REQUIRE(out.act - FL_UNARY < UNARY_ACT_COUNT && nsplit == 1, "fused_linear: activation %d on the sums of %d slices",
+                 out.act - FL_UNARY, nsplit);
+    KLLM_REQUIRE(out.act - FL_UNARY != ACT_XIELU || yout->norm_w, "fused_linear: this activation needs its two constants");
+    out.norm_w = yout->norm_w;
+  } else if (ep == FL_PARTS) {
+    out.act = 0;
+  }
   int tiles = ceil_div(m, 16);
   const bool scaled = yout->ss_in != nullptr;
   if (scaled) {

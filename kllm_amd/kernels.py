@@ -914,8 +914,11 @@ class Rope:
         self.page_size, self.heads, self.kv_heads, self.head_dim = page_size, heads, kv_heads, head_dim
 
 
+FUSED_LINEAR_UNARY = 16    # LINEAR_PARTS with act = this + an activation without a gate: see fused_linear
+
+
 def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SILU, resid=None, norm_weight=None,
-                 ss_out=None):
+                 ss_out=None, unary=None):
     """One launch for a decode batch's product of x [n, k] (bfloat16; a view
     with a row stride is taken) with w [m, k], and the step after it, by
     ``kind``: LINEAR_PARTS y float32 [nsplit, n, m]; LINEAR_SWIGLU y bfloat16
@@ -923,7 +926,9 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     cache; LINEAR_RESID adds the product to ``resid`` [n, m] float32 in place, writes
     y bfloat16 [n, m] = the new rows times ``norm_weight`` [m] and leaves partial sums of
     squares of the new rows in ``ss_out`` [n, fused_resid_parts rounded up to 4].  ``x`` may
-    be a ``ScaledRows`` (SWIGLU and ROPE): what a LINEAR_RESID product left, see there."""
+    be a ``ScaledRows`` (SWIGLU and ROPE): what a LINEAR_RESID product left, see there.
+    LINEAR_PARTS with ``unary`` = (activation without a gate, its float32 constants or None):
+    y bfloat16 [n, m] = activation(sums), one slice."""
     m, k = w.shape
     lo = _LinearOut()
     if w.dtype != torch.bfloat16:
@@ -947,7 +952,14 @@ def fused_linear(w, y, kind, x, nsplit=1, tiles_per_wg=1, rope=None, act=ACT_SIL
     if x.dim() != 2 or x.shape[1] != k or x.dtype != torch.bfloat16 or x.stride(1) != 1 or not x.is_cuda:
         raise KernelError(f"fused_linear: x {tuple(x.shape)} {x.dtype} does not fit w {tuple(w.shape)}")
     x_ptr, x_stride = x.data_ptr(), (x.stride(0) if n > 1 else k)
-    if kind == LINEAR_PARTS:
+    if kind == LINEAR_PARTS and unary is not None:
+        code, params = unary
+        if nsplit != 1 or (code == ACT_XIELU and (params is None or params.numel() != 2)):
+            raise KernelError("fused_linear: an activation on the sums takes one slice, and xielu its two constants")
+        want, dt = (n, m), torch.bfloat16
+        lo.act = FUSED_LINEAR_UNARY + int(code)
+        lo.norm_w = _ptr(params, "fused_linear activation constants", torch.float32, True)
+    elif kind == LINEAR_PARTS:
         want, dt = (nsplit, n, m), torch.float32
     elif kind == LINEAR_RESID:
         want, dt = (n, m), torch.bfloat16

@@ -13,7 +13,7 @@ import torch
 
 from .. import kernels as K
 from .base import Normed, Part, register_part
-from .linear import decode_linear, linear, linear_into, tiled_copy
+from .linear import decode_batch_fits, decode_linear, linear, linear_into, tiled_copy
 from .spec import WeightSpec
 
 
@@ -139,6 +139,10 @@ class DenseFeedForward(Part):
         if (n > 128 and self.runtime.options.get("gemm") != "library" and self.runtime.options.get("gemm_algo") is None
                 and self.hidden % (8 if xn.dtype == torch.bfloat16 else 4) == 0):
             K.gemm_act(xn, self.w_up, h, self.act, self.act_params)      # prompts: the activation in the product's epilogue
+        elif (decode_batch_fits(xn) and not self.runtime.options.get("no_fused_linear")
+              and self.runtime.options.get("gemm_algo") is None):
+            # a decode batch: the same in the decode-batch kernel's epilogue
+            h = decode_linear(ctx, xn, self.w_up, "ffn.h", self._tiled.get("up"), unary=(self.act, self.act_params))
         else:
             up = decode_linear(ctx, xn, self.w_up, "ffn.up", self._tiled.get("up"))
             K.unary_act(up, h, self.act, self.act_params)

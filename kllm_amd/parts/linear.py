@@ -277,10 +277,30 @@ def linear(ctx, x, w, tag, out_dtype=torch.float32, split=True, w_tiled=None):
     return y
 
 
-def decode_linear(ctx, x, w, tag, w_tiled=None):
+def decode_batch_fits(x):
+    """Whether a product of these rows runs on the decode-batch kernel (bfloat16, up to 16 rows,
+    all of K in a workgroup)."""
+    n, k = x.shape
+    return x.dtype == torch.bfloat16 and n <= 16 and k % 8 == 0 and K.fused_linear_fits(n, k)
+
+
+def decode_linear(ctx, x, w, tag, w_tiled=None, unary=None):
     """``linear`` for a consumer that takes float32 sums either whole or in slices: decode
-    batches of 5 to 16 rows run on the decode-batch kernel with all of K in a workgroup (one
-    result, from the tiled copy of w where there is one); everything else as ``linear`` cuts it."""
-    n = x.shape[0]
-    whole = 4 < n <= 16 and x.dtype == torch.bfloat16 and K.fused_linear_fits(n, x.shape[1])
-    return linear(ctx, x, w, tag, split=not whole, w_tiled=w_tiled)
+    batches of up to 16 rows run on the decode-batch kernel with all of K in a workgroup (one
+    result, from the tiled copy of w where there is one); everything else as ``linear`` cuts it.
+    ``unary`` = (activation without a gate, its constants): only where ``decode_batch_fits``;
+    the result is then the activation of the sums in bfloat16."""
+    n, m = x.shape[0], w.shape[0]
+    rt = ctx.runtime
+    if decode_batch_fits(x) and not rt.options.get("no_fused_linear") and rt.options.get("gemm_algo") is None:
+        tiles = 4 if m >= 16384 else 1
+        if unary is not None:
+            y = ctx.buf(tag, (n, m), torch.bfloat16)
+            K.fused_linear(w_tiled if w_tiled is not None else w, y, K.LINEAR_PARTS, x=x, tiles_per_wg=tiles, unary=unary)
+            return y
+        y = ctx.buf(tag, (1, n, m), torch.float32)
+        K.fused_linear(w_tiled if w_tiled is not None else w, y, K.LINEAR_PARTS, x=x, tiles_per_wg=tiles)
+        return y[0]
+    if unary is not None:
+        raise ValueError("decode_linear: the activation goes with the decode-batch kernel only")
+    return linear(ctx, x, w, tag)
