@@ -53,7 +53,7 @@ __device__ __forceinline__ float group4_sum(float v) {
   return v + __shfl_xor(v, 32, kWave);
 }
 
-template <int HDT, int kDecodeWaves>  // head_dim = 16 * HDT
+template <int HDT, int kDecodeWaves, bool BIASED = false>  // head_dim = 16 * HDT; BIASED: scores lose slope * distance
 __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ final_out, float* __restrict__ part,
     const bf16_t* __restrict__ cache,
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   const bool head_ok = head_in_group < G;
   const int head = kvh * G + (head_ok ? head_in_group : 0);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  const float slope = (slopes && head_ok) ? slopes[head] : 0.f;   // a bias that grows with the distance to the key
+  const float slope = (BIASED && head_ok) ? slopes[head] : 0.f;   // a bias that grows with the distance to the key
 
   bf16x8 qb[KS];
 #pragma unroll
@@ -173,7 +173,9 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = kb + 16 * u + 4 * g + i;
         const bool ok = cur.live[u] && key >= start && key < len;
-        s[u][i] = ok ? s[u][i] * scale - slope * (float)(len - 1 - key) : -INFINITY;
+        float sc = s[u][i] * scale;
+        if (BIASED) sc -= slope * (float)(len - 1 - key);      // (a constant of the code: a model without slopes has none of it)
+        s[u][i] = ok ? sc : -INFINITY;
         tmax = fmaxf(tmax, s[u][i]);
       }
     tmax = group4_max(tmax);
@@ -292,6 +294,20 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
                                        W * 16 * (16 * HDT + 4) * (int)sizeof(float));
     if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
+  }
+  if (slopes) {
+    static int raised_biased = 0;
+    if (lds > 64 * 1024 && !raised_biased) {
+      hipError_t e = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<HDT, W, true>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         W * 16 * (16 * HDT + 4) * (int)sizeof(float));
+      if (e != hipSuccess) KLLM_FAIL((int)e, "attn_decode: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      raised_biased = 1;
+    }
+    hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W, true>), grid, dim3(64 * W), lds, stream,
+                       (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, H, KV, window, scale, slopes, head_tiles, token_list);
+    return 0;
   }
   hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,

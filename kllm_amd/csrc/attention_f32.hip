@@ -221,7 +221,9 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
     for (int i = 0; i < 16; ++i) {
       const int key = kb + 8 * (i / 4) + 4 * g + i % 4;
       const bool ok = key <= my_pos && key >= my_start;
-      s[i] = ok ? s[i] * a.scale - my_slope * (float)(my_pos - key) : -INFINITY;
+      float sc = s[i] * a.scale;
+      if (a.slopes) sc -= my_slope * (float)(my_pos - key);   // (the same in every lane: a model without slopes skips it)
+      s[i] = ok ? sc : -INFINITY;
       tmax = fmaxf(tmax, s[i]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));

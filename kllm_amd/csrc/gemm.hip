@@ -172,12 +172,15 @@ __device__ __forceinline__ int mfma_swz(int row) { return (row >> 1) & 7; }
 // WR x WC waves, each with WTM x 2 MFMA tiles of 32 x 32: a workgroup's tile is 32 WTM WR rows
 // of X by 64 WC rows of W (128 x 128 with four waves, 256 x 128 and 256 x 256 with eight; for
 // decode batches 64 x 128 and 64 x 64 with two).
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
+// MODE 0: one product; 1 (DUAL): gate and up products with the gate in the epilogue; 2: one product
+// with an activation without a gate in the epilogue.
+template <typename T, typename TOUT, int MODE, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
 __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_kernel(const T* __restrict__ X,
                                                              const T* __restrict__ W,
                                                              TOUT* __restrict__ Y, int n, int m,
                                                              int k, int tiles_x, int tiles_y, int kslice, int act,
                                                              const float* __restrict__ act_params, int xcds) {
+  constexpr bool DUAL = MODE == 1;
   typedef typename MfmaOperand<T>::type op_t;   // 16 bytes of a row
   constexpr int EPC = 16 / sizeof(T);           // elements of a 16-byte chunk
   constexpr int MBK = MROW / sizeof(T);         // elements of K per stage
@@ -342,12 +345,13 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
       }
     return;
   }
-  // One product: the sums as they are, or (act >= 0) through an activation without a gate.
-  const bool has_act = act >= 0;
+  // One product: the sums as they are, or (MODE 2) through an activation without a gate.
   float a_pos = 0.f, a_neg = 0.f;
-  if (has_act && act == ACT_XIELU) {
-    a_pos = softplus_f32(act_params[0]);
-    a_neg = softplus_f32(act_params[1]);
+  if constexpr (MODE == 2) {
+    if (act == ACT_XIELU) {
+      a_pos = softplus_f32(act_params[0]);
+      a_neg = softplus_f32(act_params[1]);
+    }
   }
 #pragma unroll
   for (int i = 0; i < WTM; ++i)
@@ -358,15 +362,17 @@ __global__ __launch_bounds__(64 * WR * WC) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const long r = row0 + wr * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        const float v = acc[i][j][e];
-        if (r < n) Y[r * m + c] = from_f32<TOUT>(has_act ? unary_act(v, act, a_pos, a_neg) : v);
+        float v = acc[i][j][e];
+        if constexpr (MODE == 2) v = unary_act(v, act, a_pos, a_neg);
+        if (r < n) Y[r * m + c] = from_f32<TOUT>(v);
       }
     }
 }
 
-template <typename T, typename TOUT, bool DUAL, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
+template <typename T, typename TOUT, int MODE, int WR, int MSTAGES, int WC = 2, int WTM = 2, int WTN = 2>
 static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                             hipStream_t stream, const float* act_params = nullptr) {
+  constexpr bool DUAL = MODE == 1;
   constexpr int MBK = MROW / sizeof(T);
   constexpr int BM = 32 * WTM * WR, BN = 32 * WTN * WC;
   const int tx = ceil_div(m, DUAL ? BN / 2 : BN), ty = ceil_div(n, BM);
@@ -376,12 +382,12 @@ static int launch_mfma_tile(const void* x, const void* w, void* y, int n, int m,
   const size_t lds = (size_t)MSTAGES * (BM + BN) * MROW;
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mfma_kernel<T, TOUT, MODE, WR, MSTAGES, WC, WTM, WTN>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) KLLM_FAIL((int)e, "gemm mfma: cannot raise the LDS limit: %s", hipGetErrorString(e));
     raised = 1;
   }
-  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, DUAL, WR, MSTAGES, WC, WTM, WTN>), grid, dim3(64 * WR * WC), lds, stream,
+  hipLaunchKernelGGL((gemm_mfma_kernel<T, TOUT, MODE, WR, MSTAGES, WC, WTM, WTN>), grid, dim3(64 * WR * WC), lds, stream,
                      (const T*)x, (const T*)w, (TOUT*)y, n, m, k, tx, ty, kslice, act, act_params, xcds);
   return 0;
 }
@@ -392,9 +398,10 @@ constexpr long kNarrowBelow = 40000000;   // weights (elements) below which a de
 // they are taken when they still give every CU two rounds of work and the last round is not
 // mostly idle (8,192 x 2,560 x 2,048, two and a half rounds: 113 us against 101 us with 128 rows).  The thresholds follow
 // the chip's number of CUs.
-template <typename T, typename TOUT, bool DUAL>
+template <typename T, typename TOUT, int MODE>
 static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int k, int nsplit, int act,
                        hipStream_t stream, const float* act_params = nullptr) {
+  constexpr bool DUAL = MODE == 1;
   const int cus = device_cus();
   const int tx = ceil_div(m, DUAL ? MBN / 2 : MBN);
   // A decode batch: tiles of 64 rows, half the products and half the loads of X of 128.  In
@@ -409,13 +416,13 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
     if constexpr (!DUAL) {
       if ((long)m * k < kNarrowBelow) {
         if ((long)ceil_div(m, 64) * nsplit <= cus)
-          return launch_mfma_tile<T, TOUT, DUAL, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
-        return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+          return launch_mfma_tile<T, TOUT, MODE, 2, 3, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+        return launch_mfma_tile<T, TOUT, MODE, 2, 2, 1, 1>(x, w, y, n, m, k, nsplit, act, stream, act_params);
       }
     }
     if (sizeof(T) == 2 && (long)tx * nsplit <= cus)
-      return launch_mfma_tile<T, TOUT, DUAL, 1, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
-    return launch_mfma_tile<T, TOUT, DUAL, 1, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+      return launch_mfma_tile<T, TOUT, MODE, 1, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+    return launch_mfma_tile<T, TOUT, MODE, 1, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   }
   // 256 x 256 tiles (eight waves of 128 x 64, one workgroup a CU) fetch a third less again and
   // are 10-27 % faster (2,048 x 28,672 x 4,096: 499 us against 561 us) where their rounds fill
@@ -445,16 +452,16 @@ static int launch_mfma(const void* x, const void* w, void* y, int n, int m, int 
                            5L * mid * n >= 3L * cus * 256 * ceil_div(n, 256);
     const bool mid_fits = 100 * mid >= 85 * mid_rounds * cus || one_round;
     if (mid_fits && (!big_fits || 3 * mid_rounds <= 4 * rounds))
-      return launch_mfma_tile<T, TOUT, DUAL, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+      return launch_mfma_tile<T, TOUT, MODE, 4, 2, 2, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);
     if (big_fits)
-      return launch_mfma_tile<T, TOUT, DUAL, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+      return launch_mfma_tile<T, TOUT, MODE, 2, 2, 4, 4>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   }
   const long tall = (long)ceil_div(n, 256) * tx * nsplit;
   if (tall >= 2L * cus && 10 * tall >= 9L * ceil_div(tall, (long)cus) * cus)   // two rounds at least, nine tenths full
-    return launch_mfma_tile<T, TOUT, DUAL, 4, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+    return launch_mfma_tile<T, TOUT, MODE, 4, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
   const long tiles = (long)ceil_div(n, 128) * tx * nsplit;
-  if (tiles <= cus) return launch_mfma_tile<T, TOUT, DUAL, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);   // one per CU at most
-  return launch_mfma_tile<T, TOUT, DUAL, 2, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
+  if (tiles <= cus) return launch_mfma_tile<T, TOUT, MODE, 2, 3>(x, w, y, n, m, k, nsplit, act, stream, act_params);   // one per CU at most
+  return launch_mfma_tile<T, TOUT, MODE, 2, 2>(x, w, y, n, m, k, nsplit, act, stream, act_params);
 }
 
 // ------------------------------------------------------------------ bf16 MFMA skinny
@@ -880,8 +887,8 @@ extern "C" int kllm_gemm_act(const void* x, const void* w, void* h, int n, int m
   KLLM_REQUIRE(k % chunk == 0 && aligned16(x) && aligned16(w),
                "gemm_act: K=%d must be a multiple of %d and the operands 16-byte aligned", k, chunk);
   KLLM_REQUIRE((long)n * m < (1L << 31), "gemm_act: sizes overflow");
-  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, false>(x, w, h, n, m, k, 1, act, stream, act_params)
-                               : launch_mfma<bf16_t, bf16_t, false>(x, w, h, n, m, k, 1, act, stream, act_params))
+  if (int rc = dtype == DT_F32 ? launch_mfma<float, float, 2>(x, w, h, n, m, k, 1, act, stream, act_params)
+                               : launch_mfma<bf16_t, bf16_t, 2>(x, w, h, n, m, k, 1, act, stream, act_params))
     return rc;
   KLLM_CHECK_LAUNCH("gemm_act");
   return 0;
