@@ -23,7 +23,7 @@ Other workloads, each printing one JSON line of its own (``--model`` chooses the
                                not given)
     --kernel NAME --shape a,b,..   one kernel alone (gemm n,m,k; gemm_swiglu n,f,k; attn_prefill
                                tokens,H,KV,hd; attn_decode batch,context,H,KV,hd; add_rmsnorm n,d;
-                               copy bytes), in microseconds and against nominal and measured peaks
+                               group_norm_add n,d,groups; delta_scan tokens,H,hd; copy bytes), in microseconds and against nominal and measured peaks
     --calibrate                the box's own copy bandwidth and MFMA rates
 """
 

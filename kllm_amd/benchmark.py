@@ -428,6 +428,8 @@ def bench_kernel(name: str, shape, dtype: str = "bfloat16", reps: int = 50, warm
       attn_prefill  tokens, H, KV, hd     one prompt of that many tokens, no cached keys
       attn_decode   batch, context, H, KV, hd
       add_rmsnorm   n, d
+      group_norm_add  n, d, groups     scaled sum of two sub-layers into the stream, grouped norm
+      delta_scan    tokens, H, hd      the generalized-delta-rule recurrence of one request
       copy          bytes
 
     Returns a dict with microseconds (mean over reps), the bytes or flops the kernel must
@@ -488,6 +490,25 @@ def bench_kernel(name: str, shape, dtype: str = "bfloat16", reps: int = 50, warm
         out = torch.empty(n, d, dtype=td, device=dev)
         fn = lambda: K.add_rmsnorm(x, delta=delta, weight=w, out=out, eps=1e-5)
         nbytes = n * d * (4 + 4 + 4 + elem)
+    elif name == "group_norm_add":
+        n, d, groups = shape
+        x, w = torch.randn(n, d, device=dev), torch.ones(d, device=dev)
+        d1, d2 = torch.randn(2, n, d, device=dev), torch.randn(2, n, d, device=dev)
+        out = torch.empty(n, d, dtype=td, device=dev)
+        fn = lambda: K.group_norm_add(x, [d1, d2], mult=0.5, weight=w, out=out, groups=groups, eps=1e-5)
+        nbytes = n * d * (4 + 4 + 16 + elem)
+        note = "two sums of two slices each"
+    elif name == "delta_scan":
+        tokens, H, hd = shape
+        scan_in = torch.randn(tokens, H, K.DELTA_SCAN_FIELDS, hd, device=dev) * 0.1
+        scan_in[:, :, 3] = 0.9
+        o, state = torch.empty(tokens, H * hd, device=dev), torch.zeros(1, H, hd, hd, device=dev)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+        slots, starts, pos = i32([0]), i32([0, tokens]), i32([0])
+        fn = lambda: K.delta_scan(scan_in, o, state, slots, starts, pos, 1)
+        flops = 10.0 * tokens * H * hd * hd
+        nbytes = tokens * H * hd * (K.DELTA_SCAN_FIELDS + 1) * 4 + 2 * H * hd * hd * 4
+        note = f"{tokens} dependent steps: {{us_per_token}} us a token"
     elif name == "copy":
         (count,) = shape
         src = torch.empty(count // 4, dtype=torch.float32, device=dev).fill_(1.0)
@@ -496,11 +517,13 @@ def bench_kernel(name: str, shape, dtype: str = "bfloat16", reps: int = 50, warm
         nbytes = 2 * (count // 4) * 4
     else:
         raise ValueError(f"no kernel bench named {name!r} (gemm, gemm_swiglu, attn_prefill, attn_decode, "
-                         f"add_rmsnorm, copy)")
+                         f"add_rmsnorm, group_norm_add, delta_scan, copy)")
     for _ in range(warmup):
         fn()
     us = _event_ms(fn, reps) * 1e3
     cal = calibrate(dev)
+    if name == "delta_scan":
+        note = note.replace("{us_per_token}", f"{us / shape[0]:.3f}")
     res = {"kernel": name, "shape": list(shape), "dtype": dtype, "us": round(us, 2), "note": note}
     if flops:
         t = flops / (us * 1e-6) / 1e12

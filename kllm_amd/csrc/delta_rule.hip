@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
   const float* base = scan_in + (long)h * per_tok;
   // A block always runs its TB tokens: where the span ends before, the rest are tokens that
   // change nothing (decay one, everything else zero), so that the block's code has no branch.
-  int from[kScanStage], to[kScanStage], of_tok[kScanStage];
+  int from[kScanStage], from0[kScanStage], to[kScanStage], of_tok[kScanStage];
   float padv[kScanStage];
 #pragma unroll
   for (int k = 0; k < kScanStage; ++k) {
@@ -166,6 +166,7 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
     const int tt = idx / per_tok, e = idx % per_tok;
     of_tok[k] = tt < TB ? tt : (1 << 30);              // beyond the block: never staged
     from[k] = tt * tok_stride + e;
+    from0[k] = e;                                      // the same element of the block's first token
     to[k] = tt < TB ? tt * VEC + (e / hd) * HP + e % hd : 0;
     padv[k] = e / hd == 3 ? 1.f : 0.f;
   }
@@ -174,10 +175,13 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
   // one block's arithmetic does not.
   float set0[kScanStage], set1[kScanStage], set2[kScanStage];
   auto ask = [&](float (&pre)[kScanStage], int first) {           // the block's elements into registers
+    // Every load is made, none inside a branch (the compiler then counts the loads in flight and
+    // a later wait is for these alone): an element of a token that does not exist reads a place
+    // that does, and is dropped when the block is put into LDS.
     const int count = min(TB, t1 - first);                         // <= 0: there is no such block
-    const float* src = base + (long)first * tok_stride;
+    const float* src = base + (long)min(first, t1 - 1) * tok_stride;
 #pragma unroll
-    for (int k = 0; k < kScanStage; ++k) pre[k] = (of_tok[k] < count) ? src[from[k]] : 0.f;
+    for (int k = 0; k < kScanStage; ++k) pre[k] = src[of_tok[k] < count ? from[k] : from0[k]];
   };
   auto put = [&](const float (&pre)[kScanStage], float* buf, int first) {
     const int count = min(TB, t1 - first);
@@ -250,7 +254,13 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
     if (col && p < count) o_out[(long)(tb + p) * o_step + h * hd + j] = o_keep;
     put(next, tok + (which ^ 1) * TB * VEC, tb + TB);
     ask(next, tb + 4 * TB);
-    __syncthreads();                                   // the next block is staged; this one is done with
+    // The next block is staged; this one is done with.  The barrier orders LDS traffic only: it
+    // waits for LDS (lgkmcnt 0) and leaves the loads from memory in flight, which a
+    // __syncthreads() would wait for, every block paying the memory's latency.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   };
   for (int tb = t0; tb < t1; tb += 3 * TB) {           // the three sets of registers take turns by name
     block(tb, set1);
@@ -323,19 +333,27 @@ extern "C" int kllm_delta_scan(const float* scan_in, float* o_out, float* state,
   KLLM_REQUIRE(scan_in && o_out && state && slots && span_start && span_pos, "delta_scan: null pointer");
   KLLM_REQUIRE(n_spans > 0 && H > 0 && H <= 65535 && hd > 0 && hd <= 256, "delta_scan: bad sizes spans=%d H=%d hd=%d",
                n_spans, H, hd);
-  // a column's rows in fours over neighbouring lanes: 4, 8, 16 ... 256 rows with padding
+  // A column's rows over neighbouring lanes, four to a lane for heads up to 64 and eight above
+  // (sixteen lanes sum by data-parallel moves alone; more need a lane exchange through LDS on
+  // the chain from token to token): 4, 8 ... 64 rows with padding, then 128, 256.
+  const int nr = hd > 64 ? 8 : 4;
   int parts = 1;
-  while (parts * 4 < hd) parts *= 2;
+  while (parts * nr < hd) parts *= 2;
   const int cols = kScanThreads / parts;
   const dim3 grid(n_spans, H, ceil_div(hd, cols));
-#define KLLM_SCAN(PARTS)                                                                                          \
-  case PARTS:                                                                                                     \
-    hipLaunchKernelGGL((delta_scan_kernel<PARTS, 4>), grid, dim3(kScanThreads), 0, stream, scan_in, o_out, state, \
-                       slots, span_start, span_pos, H, hd);                                                       \
-    break
-  switch (parts) {
-    KLLM_SCAN(1); KLLM_SCAN(2); KLLM_SCAN(4); KLLM_SCAN(8); KLLM_SCAN(16); KLLM_SCAN(32); KLLM_SCAN(64);
-    default: KLLM_FAIL(ERR_ARG, "delta_scan: heads of %d are not built", hd);
+#define KLLM_SCAN(PARTS, NR)                                                                                       \
+  hipLaunchKernelGGL((delta_scan_kernel<PARTS, NR>), grid, dim3(kScanThreads), 0, stream, scan_in, o_out, state, \
+                     slots, span_start, span_pos, H, hd)
+  if (nr == 4) {
+    switch (parts) {
+      case 1: KLLM_SCAN(1, 4); break;
+      case 2: KLLM_SCAN(2, 4); break;
+      case 4: KLLM_SCAN(4, 4); break;
+      case 8: KLLM_SCAN(8, 4); break;
+      default: KLLM_SCAN(16, 4); break;
+    }
+  } else {
+    if (parts <= 16) KLLM_SCAN(16, 8); else KLLM_SCAN(32, 8);
   }
 #undef KLLM_SCAN
   KLLM_CHECK_LAUNCH("delta_scan");

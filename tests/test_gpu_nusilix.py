@@ -92,6 +92,29 @@ def test_xielu_with_its_learned_constants(dtype):
         assert rel(out.float().cpu(), want) < (1e-6 if dtype == "float32" else 5e-3)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n", [3, 16, 200])
+def test_the_activation_in_a_products_epilogue(n, dtype):
+    """x . w^T through xIELU in the tiled product's epilogue (any rows) and, in bfloat16, in the
+    decode-batch kernel's (up to 16 rows, from the tiled copy of the weights)."""
+    from kllm_amd import kernels as K
+    g = torch.Generator().manual_seed(n)
+    k, m = 96, 200
+    x, w = torch.randn(n, k, generator=g), torch.randn(m, k, generator=g) / math.sqrt(k)
+    params = torch.tensor([0.4, -0.3])
+    xd, wd = dev(x, TD[dtype]), dev(w, TD[dtype])
+    want = P.xielu(xd.double().cpu() @ wd.double().cpu().T, 0.4, -0.3)
+    tol = 1e-5 if dtype == "float32" else 6e-3
+    h = torch.empty(n, m, device="cuda", dtype=TD[dtype])
+    K.gemm_act(xd, wd, h, K.ACT_XIELU, dev(params))
+    assert rel(h.float().cpu(), want) < tol
+    if dtype == "bfloat16" and n <= 16:
+        for weights in (wd, K.fused_linear_tile(wd, K.LINEAR_PARTS)):
+            h2 = torch.zeros(n, m, device="cuda", dtype=torch.bfloat16)
+            K.fused_linear(weights, h2, K.LINEAR_PARTS, x=xd, unary=(K.ACT_XIELU, dev(params)))
+            assert rel(h2.float().cpu(), want) < tol
+
+
 class HandCache:
     """A paged cache of one layer and its tables, filled by hand: ``lengths`` requests whose
     pages are handed out in a shuffled order."""
