@@ -500,7 +500,7 @@ def bench_kernel(name: str, shape, dtype: str = "bfloat16", reps: int = 50, warm
         note = "two sums of two slices each"
     elif name == "delta_scan":
         tokens, H, hd = shape
-        scan_in = torch.randn(tokens, H, K.DELTA_SCAN_FIELDS, hd, device=dev) * 0.1
+        scan_in = torch.randn(H, tokens, K.DELTA_SCAN_FIELDS, hd, device=dev) * 0.1
         scan_in[:, :, 3] = 0.9
         o, state = torch.empty(tokens, H * hd, device=dev), torch.zeros(1, H, hd, hd, device=dev)
         i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)

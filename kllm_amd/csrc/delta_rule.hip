@@ -22,7 +22,7 @@ constexpr int kPrepThreads = 256;
 constexpr int kScanFields = 6;
 
 // proj: [nsplit][n][5*HD + L], columns r | k | v | g | a | w1.
-// scan_in: [n][H][6][hd]; gate: [n][HD] = sigmoid(g).
+// scan_in: [H][n][6][hd] (a head's tokens follow each other, as the scan reads them); gate: [n][HD] = sigmoid(g).
 // A workgroup takes one token and as many whole heads as its threads hold channels
 // (blockIdx.y), a thread one channel: every load of a thread is independent of the others.
 template <typename TW>
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kPrepThreads) void delta_prep_kernel(
   const float w = expf(-decay_scale * sigmoid_f32(lr));
   const float a = sigmoid_f32(f[4] + ab);
   const float u = f[1] / sqrtf(kss + key_eps);
-  float* o = scan_in + (((long)t * H + h) * kScanFields) * hd + e;
+  float* o = scan_in + (((long)h * gridDim.x + t) * kScanFields) * hd + e;
   o[0 * hd] = f[0];
   o[1 * hd] = f[1];
   o[2 * hd] = f[2];
@@ -115,29 +115,35 @@ __device__ __forceinline__ float parts_sum(float v) {
 }
 
 constexpr int kScanThreads = 256;
-constexpr int kScanStage = 12;            // elements of a block that a thread stages, at most
+constexpr int kScanWaves = kScanThreads / kWave;
 
 // The recurrence.  Columns of the state (value channels) do not see each other, so a workgroup
 // takes a block of columns of one (span, head): thread (j, p) holds rows [NR p, NR p + NR) of
 // column j, the PARTS threads of a column are neighbouring lanes of one wave.  A token's vectors
-// are the same for every column; they are staged through LDS, a block of tokens at a time and
-// the next block's loads in flight while this block's tokens are worked through, so that the
-// chain from token to token holds arithmetic and LDS reads only.  Rows beyond hd are padding:
-// their vectors are zero in LDS and their state stays zero.
+// are the same for every column; they are staged through LDS a block of tokens at a time (32
+// tokens for heads up to 64): the next block's loads from memory are all asked for before this
+// block's tokens are worked through and put into LDS behind them, so the memory's latency hides
+// behind a block's arithmetic (it did not behind 8 tokens'), and the chain from token to token
+// holds arithmetic and LDS reads only.  A block's code has no branch: a span that ends inside
+// a block is filled with tokens that change nothing (decay one, everything else zero).  Rows
+// beyond hd are padding: their vectors are zero in LDS and their state stays zero.
 template <int PARTS, int NR>
 __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
     const float* __restrict__ scan_in, float* __restrict__ o_out, float* __restrict__ state,
-    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos, int H,
-    int hd) {
+    const int* __restrict__ slots, const int* __restrict__ span_start, const int* __restrict__ span_pos, int n,
+    int H, int hd) {
   static_assert(NR % 4 == 0, "rows in fours");
   constexpr int HP = PARTS * NR;                       // rows with padding
   constexpr int COLS = kScanThreads / PARTS;           // columns of a workgroup
-  constexpr int TB0 = HP >= 512 ? 1 : 512 / HP;
-  constexpr int TB = TB0 < PARTS ? TB0 : PARTS;        // tokens of a block: lane p of a column keeps token p's output
+  constexpr int TB = 2048 / HP < 32 ? 2048 / HP : 32;  // tokens of a block
+  constexpr int KEEPS = (TB + PARTS - 1) / PARTS;      // outputs a lane keeps: token tt's lies in lane tt % PARTS
   constexpr int VEC = kScanFields * HP;                // floats of a token in LDS
-  static_assert(kScanStage * kScanThreads >= TB * VEC, "a block is staged whole");
-  __shared__ __attribute__((aligned(16))) float tok[2 * TB * VEC];
+  constexpr int EPL = (VEC + kWave - 1) / kWave;       // elements of a token that a lane stages
+  constexpr int TPW = TB / kScanWaves;                 // tokens of a block that a wave stages
+  static_assert(TB % kScanWaves == 0 && TB * VEC * sizeof(float) <= 48 * 1024, "a block is staged by whole waves");
+  __shared__ __attribute__((aligned(16))) float tok[TB * VEC];
   const int span = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid % kWave, wave = tid / kWave;
   const int j = blockIdx.z * COLS + tid / PARTS, p = tid % PARTS;
   const bool col = j < hd;
   const int row0 = p * NR;
@@ -151,53 +157,56 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
     s[i] = (col && r < hd && !fresh) ? S[(long)r * hd + j] : 0.f;
   }
   if (HP != hd)
-    for (int i = tid; i < 2 * TB * VEC; i += kScanThreads) tok[i] = 0.f;
-  // Where this thread's elements of a block come from and go to: worked out once.
+    for (int i = tid; i < TB * VEC; i += kScanThreads) tok[i] = 0.f;
+  // Staging: wave w takes the block's tokens w, w + 4, ...; a lane the elements lane, lane + 64,
+  // ... of a token.  Where an element goes in LDS, and what stands there for a token that does
+  // not exist, is worked out once.
   const int per_tok = kScanFields * hd;                // floats of a token in memory
-  const int tok_stride = H * per_tok;
-  const float* base = scan_in + (long)h * per_tok;
-  // A block always runs its TB tokens: where the span ends before, the rest are tokens that
-  // change nothing (decay one, everything else zero), so that the block's code has no branch.
-  int from[kScanStage], from0[kScanStage], to[kScanStage], of_tok[kScanStage];
-  float padv[kScanStage];
+  const long tok_stride = per_tok;                     // a head's tokens follow each other
+  const float* base = scan_in + (long)h * n * per_tok;
+  int from_e[EPL], to_e[EPL];
+  float pad_e[EPL];
 #pragma unroll
-  for (int k = 0; k < kScanStage; ++k) {
-    const int idx = tid + k * kScanThreads;
-    const int tt = idx / per_tok, e = idx % per_tok;
-    of_tok[k] = tt < TB ? tt : (1 << 30);              // beyond the block: never staged
-    from[k] = tt * tok_stride + e;
-    from0[k] = e;                                      // the same element of the block's first token
-    to[k] = tt < TB ? tt * VEC + (e / hd) * HP + e % hd : 0;
-    padv[k] = e / hd == 3 ? 1.f : 0.f;
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + i * kWave;
+    from_e[i] = e < per_tok ? e : 0;                   // (an element beyond the token reads a place that exists)
+    to_e[i] = e < per_tok ? (e / hd) * HP + e % hd : -1;
+    pad_e[i] = e / hd == 3 ? 1.f : 0.f;
   }
-  // Blocks on their way from memory wait in three sets of registers that take turns by name: a
-  // block is asked for three blocks ahead of its use, which covers the memory's latency where
-  // one block's arithmetic does not.
-  float set0[kScanStage], set1[kScanStage], set2[kScanStage];
-  auto ask = [&](float (&pre)[kScanStage], int first) {           // the block's elements into registers
-    // Every load is made, none inside a branch (the compiler then counts the loads in flight and
-    // a later wait is for these alone): an element of a token that does not exist reads a place
-    // that does, and is dropped when the block is put into LDS.
-    const int count = min(TB, t1 - first);                         // <= 0: there is no such block
-    const float* src = base + (long)min(first, t1 - 1) * tok_stride;
+  float pre[TPW * EPL];
+  // Every load is made, none inside a branch: an element of a token that does not exist reads a
+  // token that does, and is dropped when the block is put into LDS.
+  auto ask = [&](int first) {
 #pragma unroll
-    for (int k = 0; k < kScanStage; ++k) pre[k] = src[of_tok[k] < count ? from[k] : from0[k]];
+    for (int q = 0; q < TPW; ++q) {
+      const int t = min(first + wave + q * kScanWaves, t1 - 1);
+      const float* src = base + (long)t * tok_stride;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) pre[q * EPL + i] = src[from_e[i]];
+    }
   };
-  auto put = [&](const float (&pre)[kScanStage], float* buf, int first) {
-    const int count = min(TB, t1 - first);
+  auto put = [&](int first) {
 #pragma unroll
-    for (int k = 0; k < kScanStage; ++k)
-      if (of_tok[k] < TB) buf[to[k]] = of_tok[k] < count ? pre[k] : padv[k];
+    for (int q = 0; q < TPW; ++q) {
+      const int tt = wave + q * kScanWaves;
+      const bool there = first + tt < t1;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i)
+        if (to_e[i] >= 0) tok[tt * VEC + to_e[i]] = there ? pre[q * EPL + i] : pad_e[i];
+    }
+  };
+  auto lds_barrier = [&]() {   // orders LDS traffic only: loads from memory stay in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   };
   __syncthreads();                                     // the padding is zero before anything is staged
-  ask(set0, t0);
-  ask(set1, t0 + TB);
-  ask(set2, t0 + 2 * TB);
-  put(set0, tok, t0);
-  ask(set0, t0 + 3 * TB);
+  ask(t0);
+  put(t0);
   __syncthreads();
   const long o_step = (long)H * hd;
-  float o_keep = 0.f;                                  // lane p of a column: the output of the block's token p
+  float o_keep[KEEPS];
   struct TokenVectors {                                // this thread's rows of a token's vectors
     floatx4 u[NR / 4], w[NR / 4], k[NR / 4], a[NR / 4], r[NR / 4];
     float vj;
@@ -235,39 +244,25 @@ __global__ __launch_bounds__(kScanThreads) void delta_scan_kernel(
         if (e % 2 == 0) o0 = fmaf(sn, T.r[c][e], o0); else o1 = fmaf(sn, T.r[c][e], o1);
       }
     const float o_sum = parts_sum<PARTS>(o0 + o1);     // not part of the chain from token to token
-    o_keep = p == tt ? o_sum : o_keep;
+    o_keep[tt / PARTS] = p == tt % PARTS ? o_sum : o_keep[tt / PARTS];
   };
-  // Block `tb` is worked through from its LDS buffer, a token's vectors read while the token
-  // before it is worked on; then the next block goes from its registers into the other buffer
-  // and those registers are asked for the block three further on.
-  auto block = [&](int tb, float (&next)[kScanStage]) {
-    const int count = min(TB, t1 - tb);
-    const int which = ((tb - t0) / TB) & 1;            // the two LDS buffers take turns
-    const float* buf = tok + which * TB * VEC;
-    TokenVectors cur = fetch(buf);
+  for (int tb = t0; tb < t1; tb += TB) {
+    ask(tb + TB);                                      // the next block, on its way during this one
+    TokenVectors cur = fetch(tok);
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
-      const TokenVectors nxt = fetch(buf + (tt + 1 < TB ? tt + 1 : tt) * VEC);
+      const TokenVectors nxt = fetch(tok + (tt + 1 < TB ? tt + 1 : tt) * VEC);
       token(tt, cur);
       cur = nxt;
     }
-    if (col && p < count) o_out[(long)(tb + p) * o_step + h * hd + j] = o_keep;
-    put(next, tok + (which ^ 1) * TB * VEC, tb + TB);
-    ask(next, tb + 4 * TB);
-    // The next block is staged; this one is done with.  The barrier orders LDS traffic only: it
-    // waits for LDS (lgkmcnt 0) and leaves the loads from memory in flight, which a
-    // __syncthreads() would wait for, every block paying the memory's latency.
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-  };
-  for (int tb = t0; tb < t1; tb += 3 * TB) {           // the three sets of registers take turns by name
-    block(tb, set1);
-    if (tb + TB >= t1) break;
-    block(tb + TB, set2);
-    if (tb + 2 * TB >= t1) break;
-    block(tb + 2 * TB, set0);
+#pragma unroll
+    for (int q = 0; q < KEEPS; ++q) {
+      const int t = tb + q * PARTS + p;
+      if (col && q * PARTS + p < TB && t < t1) o_out[(long)t * o_step + h * hd + j] = o_keep[q];
+    }
+    lds_barrier();                                     // everybody is done with this block
+    put(tb + TB);
+    lds_barrier();                                     // the next block is staged
   }
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
@@ -328,8 +323,9 @@ extern "C" int kllm_delta_prep(const float* proj, int nsplit, long split_stride,
 extern "C" int kllm_delta_scan_max_dim(void) { return 256; }
 
 extern "C" int kllm_delta_scan(const float* scan_in, float* o_out, float* state, const int* slots,
-                               const int* span_start, const int* span_pos, int n_spans, int H, int hd,
+                               const int* span_start, const int* span_pos, int n_spans, int n, int H, int hd,
                                hipStream_t stream) {
+  KLLM_REQUIRE(n > 0, "delta_scan: no tokens");
   KLLM_REQUIRE(scan_in && o_out && state && slots && span_start && span_pos, "delta_scan: null pointer");
   KLLM_REQUIRE(n_spans > 0 && H > 0 && H <= 65535 && hd > 0 && hd <= 256, "delta_scan: bad sizes spans=%d H=%d hd=%d",
                n_spans, H, hd);
@@ -343,7 +339,7 @@ extern "C" int kllm_delta_scan(const float* scan_in, float* o_out, float* state,
   const dim3 grid(n_spans, H, ceil_div(hd, cols));
 #define KLLM_SCAN(PARTS, NR)                                                                                       \
   hipLaunchKernelGGL((delta_scan_kernel<PARTS, NR>), grid, dim3(kScanThreads), 0, stream, scan_in, o_out, state, \
-                     slots, span_start, span_pos, H, hd)
+                     slots, span_start, span_pos, n, H, hd)
   if (nr == 4) {
     switch (parts) {
       case 1: KLLM_SCAN(1, 4); break;

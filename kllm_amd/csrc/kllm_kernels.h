@@ -313,9 +313,9 @@ int kllm_qk_norm_append(const float* qk, int nsplit, long split_stride, const fl
  * o = S^T r, u = k / sqrt(sum k^2 + key_eps).
  * prep: proj [nsplit][n][5*H*hd + L] holds the sums of the products r | k | v | g | a | w1;
  *   w = exp(-decay_scale * sigmoid(w2 tanh(w1) + w0)), a = sigmoid(a + a_bias); writes scan_in
- *   [n][H][6][hd] (r, k, v, w, u, a*u) and gate [n][H*hd] = sigmoid(g).  w2 is [H*hd][L] in w_dtype;
+ *   [H][n][6][hd] (r, k, v, w, u, a*u; a head's tokens follow each other) and gate [n][H*hd] = sigmoid(g).  w2 is [H*hd][L] in w_dtype;
  *   with `low` (sums [low_nsplit][n][H*hd] of w2 tanh(w1), made by a matrix kernel) it is not read.
- * scan: one request after the other through state [slots][H][hd][hd] (float32; zero at
+ * scan: the n tokens of n_spans requests, each request through its state [slots][H][hd][hd] (float32; zero at
  *   position 0), o_out [n][H*hd]; hd up to kllm_delta_scan_max_dim().
  * out: out[n][H*hd] = o / sqrt(mean over the head of o^2 + eps) * weight * gate. */
 int kllm_delta_prep(const float* proj, int nsplit, long split_stride, const float* a_bias, const void* w2,
@@ -324,7 +324,7 @@ int kllm_delta_prep(const float* proj, int nsplit, long split_stride, const floa
                     hipStream_t stream);
 int kllm_delta_scan_max_dim(void);
 int kllm_delta_scan(const float* scan_in, float* o_out, float* state, const int* slots,
-                    const int* span_start, const int* span_pos, int n_spans, int H, int hd,
+                    const int* span_start, const int* span_pos, int n_spans, int n, int H, int hd,
                     hipStream_t stream);
 int kllm_delta_out(const float* o, const float* gate, const float* weight, float eps, void* out, int n, int H,
                    int hd, int dtype, hipStream_t stream);

@@ -136,7 +136,7 @@ def _declare(lib):
         "kllm_qk_norm_append": [P, I, L, P, P, P, P, F, F, I, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "kllm_delta_prep": [P, I, L, P, P, P, P, I, L, F, F, P, P, I, I, I, I, I, P],
         "kllm_delta_scan_max_dim": [],
-        "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, P],
+        "kllm_delta_scan": [P, P, P, P, P, P, I, I, I, I, P],
         "kllm_delta_out": [P, P, P, F, P, I, I, I, I, P],
     }
     for name, args in sigs.items():
@@ -1278,14 +1278,14 @@ def delta_scan_max_dim() -> int:
 
 def delta_prep(proj, a_bias, w2, w0, decay_scale, key_eps, scan_in, gate, heads, head_dim, low=None):
     """proj: float32 sums [nsplit, n, 5*H*hd + L] of the products r | k | v | g | a | w1; writes
-    what the recurrence reads, scan_in [n, H, 6, hd], and gate [n, H*hd] = sigmoid(g).  ``low``:
+    what the recurrence reads, scan_in [H, n, 6, hd], and gate [n, H*hd] = sigmoid(g).  ``low``:
     float32 sums [slices, n, H*hd] of w2 . tanh(w1 part) where a matrix kernel made them (the
     kernel then leaves that product alone)."""
     n, HD = gate.shape
     L = w2.shape[1]
     nsplit, stride = _splits(proj, n, 5 * HD + L, "delta_prep")
     low_ns, low_st = _splits(low, n, HD, "delta_prep low") if low is not None else (0, 0)
-    if (HD != heads * head_dim or tuple(scan_in.shape) != (n, heads, DELTA_SCAN_FIELDS, head_dim)
+    if (HD != heads * head_dim or tuple(scan_in.shape) != (heads, n, DELTA_SCAN_FIELDS, head_dim)
             or w2.shape[0] != HD or a_bias.numel() != HD or w0.numel() != HD):
         raise KernelError("delta_prep: shapes do not fit")
     F32 = torch.float32
@@ -1296,9 +1296,9 @@ def delta_prep(proj, a_bias, w2, w0, decay_scale, key_eps, scan_in, gate, heads,
 
 
 def delta_scan(scan_in, o_out, state, slots, span_start, span_pos, n_spans):
-    """The recurrence, one request after the other: scan_in [n, H, 6, hd], o_out [n, H*hd], state
+    """The recurrence, each request through its state: scan_in [H, n, 6, hd], o_out [n, H*hd], state
     [slots, H, hd, hd] float32 (started from zero where a span's position is 0)."""
-    n, H, _, hd = scan_in.shape
+    H, n, _, hd = scan_in.shape
     if (tuple(o_out.shape) != (n, H * hd) or tuple(state.shape[1:]) != (H, hd, hd) or state.dtype != torch.float32
             or slots.numel() < n_spans or span_start.numel() < n_spans + 1 or span_pos.numel() < n_spans):
         raise KernelError("delta_scan: shapes do not fit")
@@ -1306,7 +1306,7 @@ def delta_scan(scan_in, o_out, state, slots, span_start, span_pos, n_spans):
     _launch("kllm_delta_scan", "delta_scan", _ptr(scan_in, "delta_scan in", F32), _ptr(o_out, "delta_scan out", F32),
             _ptr(state, "delta_scan state", F32), _ptr(slots, "delta_scan slots", I32),
             _ptr(span_start, "delta_scan span_start", I32), _ptr(span_pos, "delta_scan span_pos", I32),
-            int(n_spans), H, hd, _stream())
+            int(n_spans), n, H, hd, _stream())
 
 
 def delta_out(o, gate, weight, eps, out, heads, head_dim):

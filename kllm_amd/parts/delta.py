@@ -97,7 +97,7 @@ class GeneralDeltaMixer(Part):
             t = ctx.buf("delta.tanh", (n, rank), self.runtime.dtype)
             K.unary_act(proj, t, K.ACT_TANH, first_column=5 * self.width)
             low = linear(ctx, t, self.w2, "delta.low")
-        scan_in = ctx.buf("delta.scan_in", (n, self.heads, K.DELTA_SCAN_FIELDS, self.head_dim), f32)
+        scan_in = ctx.buf("delta.scan_in", (self.heads, n, K.DELTA_SCAN_FIELDS, self.head_dim), f32)
         gate = ctx.buf("delta.gate", (n, self.width), f32)
         K.delta_prep(proj, self.a_bias, self.w2, self.w0, self.decay_scale, self.key_eps, scan_in, gate,
                      self.heads, self.head_dim, low=low)

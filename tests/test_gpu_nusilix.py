@@ -267,7 +267,7 @@ def test_delta_rule_kernels_carry_their_state_and_start_a_used_slot_from_zero(H,
         x = torch.cat([hs[s][a:b] for s, a, b in step]).double()
         sums = (x @ w_in.T).float()
         n = sums.shape[0]
-        scan_in = torch.empty(n, H, K.DELTA_SCAN_FIELDS, hd, device="cuda")
+        scan_in = torch.empty(H, n, K.DELTA_SCAN_FIELDS, hd, device="cuda")
         gate, o = torch.empty(n, HD, device="cuda"), torch.empty(n, HD, device="cuda")
         K.delta_prep(dev(torch.stack([sums * 0.5, sums * 0.5])), dev(w["a.b"]), dev(w["w2"], TD[dtype]), dev(w["w0"]),
                      math.exp(-0.5), 1e-6, scan_in, gate, H, hd)
