@@ -327,9 +327,9 @@ def nusilix_config(width, heads, kv_heads, head_dim, ff, layers, vocab, delta_ev
         else:
             entries.append({"type": "attention", "mlp": mlp,
                             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim,
-                                      "scale": head_dim ** -0.5, "q_temp": {"coef": 0.3, "every": 256}}})
-    return {"architecture": "Nusilix", "vocab": vocab, "width": width, "residual_mult": 0.5,
-            "norm": {"eps": 1e-6, "groups": 2}, "layers": entries}
+                                      "scale": head_dim ** -0.5, "q_temp": {"coef": 0.2, "every": 512}}})
+    return {"architecture": "Nusilix", "vocab": vocab, "width": width, "residual_mult": 0.7,
+            "norm": {"eps": 1e-5, "groups": 4}, "layers": entries}
 
 
 def llama_config(width, heads, kv_heads, head_dim, ff, layers, vocab) -> dict:

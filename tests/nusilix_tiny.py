@@ -25,7 +25,7 @@ import torch
 import plain_nusilix as P
 
 
-def attn(heads, kv, dim, coef=0.3, every=8, scale=None, ff=None):
+def attn(heads, kv, dim, coef=0.35, every=8, scale=None, ff=None):
     return {"type": "attention",
             "mixer": {"dim": dim, "vdim": dim, "heads": heads, "kv_heads": kv, "scale": scale or dim ** -0.5 * 1.5,
                       "q_temp": {"coef": coef, "every": every}},
@@ -44,7 +44,7 @@ def _cfg(vocab, width, layers, eps, groups, mult):
 
 CONFIGS = {
     "N1": _cfg(96, 64, [attn(4, 2, 16, ff=80), delta(2, 16, rank=8, ff=72), attn(4, 2, 16, every=5, ff=80)],
-               1e-5, 2, 0.5),
+               1e-5, 2, 0.45),
     "N2": _cfg(128, 128, [delta(2, 32, rank=16, ff=96), attn(4, 1, 64, coef=0.5, every=8),
                           attn(4, 1, 64, coef=0.5, every=8, ff=160)], 1e-6, 1, 1.0),
     "N3": _cfg(101, 96, [attn(8, 1, 32, every=16, ff=64), delta(1, 64, rank=12, ff=56),

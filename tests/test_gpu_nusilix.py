@@ -51,7 +51,7 @@ def test_sinusoidal_positions_far_out():
         assert (x.cpu().double() - 1 - P.sinusoid(pos, d)).abs().max() < 2e-7
 
 
-@pytest.mark.parametrize("d,groups", [(64, 1), (64, 2), (96, 3), (72, 4), (320, 2), (2048, 1), (4096, 8), (24, 24)])
+@pytest.mark.parametrize("d,groups", [(64, 1), (64, 2), (96, 3), (72, 4), (288, 2), (2048, 1), (4096, 8), (24, 24)])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_group_norm_adds_a_scaled_sum_and_normalises_in_groups(d, groups, dtype):
     from kllm_amd import kernels as K
@@ -144,7 +144,7 @@ def spans_context(lens, starts_pos):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,KV,hd", [(4, 2, 16), (4, 1, 64), (8, 1, 32), (2, 2, 128), (6, 3, 24), (8, 2, 48)])
+@pytest.mark.parametrize("H,KV,hd", [(4, 2, 16), (4, 1, 64), (8, 1, 32), (2, 2, 128), (6, 3, 24), (10, 2, 80)])
 def test_keys_as_values_attention_kernels_with_a_far_key(H, KV, hd, dtype):
     """Queries and keys go through the norm-and-append kernel in portions, then every attention
     kernel that takes the sizes reads the pages.  Key 3 of the long request is made to point
