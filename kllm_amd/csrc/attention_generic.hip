@@ -9,7 +9,13 @@
 // scores of a row in shared memory, scores are taken 256 keys at a time with
 // a running maximum and sum, so the context is not bounded by a buffer.
 //
-// Page layout, per page and KV head: keys [slot][hd], values [hd][slot].
+// Options that a design may ask for: values of another width than the keys
+// (vd); a chunked mask (chunk > 0: the query at p reads no key before
+// p - p % chunk, chunks counted from position 0 of the request); a sink
+// (sink != 0: the softmax's denominator has one more term, exp(0), a key whose
+// score is 0 and whose value is nothing).
+//
+// Page layout: keys [KV][slot][hd], then values [KV][vd][slot].
 #include <math.h>
 
 #include "common.hpp"
@@ -25,7 +31,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
     const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int hd,
-    int window, float scale, const float* __restrict__ slopes) {
+    int vd, int window, int chunk, int sink, float scale, const float* __restrict__ slopes) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[kAttnThreads];
   __shared__ float red[16];
@@ -36,17 +42,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
   const int pos = positions[t];
   const int len = pos + 1;
   const float slope = slopes ? slopes[h] : 0.f;   // a bias that grows with the distance to the key
-  const int start = (window > 0 && len > window) ? len - window : 0;
+  const int start = first_key(pos, window, chunk);
   const int* table = block_table + (long)span_of_token[t] * max_pages;
-  const long block = (long)page_size * hd;
+  const long kblock = (long)page_size * hd, vblock = (long)page_size * vd;
+  const long page_elems = (long)KV * (kblock + vblock);
 
   const T* qrow = q + ((long)t * H + h) * hd;
   for (int i = tid; i < hd; i += kAttnThreads) qs[i] = to_f32(qrow[i]);
   __syncthreads();
 
   // Values: thread (d, sl) sums over the pages sl, sl + nslice, ... of a chunk.
-  const int nslice = kAttnThreads / hd;
-  const int d = tid % hd, sl = tid / hd;
+  const int nslice = kAttnThreads / vd;
+  const int d = tid % vd, sl = tid / vd;
   const bool pv_thread = sl < nslice;
 
   const int chunk_pages = page_size >= kAttnThreads ? 1 : kAttnThreads / page_size;
@@ -60,7 +67,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     const int key = base + tid;
     if (tid < chunk_keys && key >= start && key < len) {
       const int page = table[key / page_size];
-      const T* krow = cache + (((long)page * 2 + 0) * KV + kvh) * block + (long)(key % page_size) * hd;
+      const T* krow = cache + page * page_elems + kvh * kblock + (long)(key % page_size) * hd;
       float dot = 0.f;
       for (int i = 0; i < hd; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
       s = dot * scale - slope * (float)(pos - key);
@@ -81,7 +88,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
         const int lo = max(start - pbase, 0), hi = min(len - pbase, page_size);
         if (lo >= hi) continue;
         const int page = table[pbase / page_size];
-        const T* vrow = cache + (((long)page * 2 + 1) * KV + kvh) * block + (long)d * page_size;
+        const T* vrow = cache + page * page_elems + KV * kblock + kvh * vblock + (long)d * page_size;
         const float* pp = ps + pg * page_size;
         for (int sidx = lo; sidx < hi; ++sidx) acc = fmaf(pp[sidx], to_f32(vrow[sidx]), acc);
       }
@@ -89,12 +96,18 @@ __global__ __launch_bounds__(kAttnThreads) void attn_generic_kernel(
     __syncthreads();  // ps is rewritten by the next chunk
   }
 
+  if (sink) {   // one more key whose score is 0: it joins the sum, and nothing else
+    const float m_all = fmaxf(m, 0.f);
+    const float alpha = expf(m - m_all);
+    l = l * alpha + expf(-m_all);
+    acc *= alpha;
+  }
   part[tid] = pv_thread ? acc : 0.f;
   __syncthreads();
-  if (tid < hd) {
+  if (tid < vd) {
     float o = 0.f;
-    for (int s2 = 0; s2 < nslice; ++s2) o += part[s2 * hd + tid];
-    out[((long)t * H + h) * hd + tid] = from_f32<T>(o / l);
+    for (int s2 = 0; s2 < nslice; ++s2) o += part[s2 * vd + tid];
+    out[((long)t * H + h) * vd + tid] = from_f32<T>(o / l);
   }
 }
 
@@ -104,8 +117,9 @@ using namespace kllm;
 
 extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                                  const int* span_of_token, const int* block_table, int max_pages,
-                                 int page_size, int n, int H, int KV, int hd, int window,
-                                 float scale, const float* slopes, int dtype, hipStream_t stream) {
+                                 int page_size, int n, int H, int KV, int hd, int vd, int window,
+                                 int chunk, int sink, float scale, const float* slopes, int dtype,
+                                 hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && positions && span_of_token && block_table,
                "attn_generic: null pointer");
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_generic: bad heads n=%d H=%d KV=%d", n,
@@ -114,18 +128,19 @@ extern "C" int kllm_attn_generic(const void* q, void* out, const void* cache, co
                kMaxHeadDim);
   KLLM_REQUIRE(page_size > 0 && page_size <= kAttnThreads && max_pages > 0,
                "attn_generic: page_size %d is outside [1, %d]", page_size, kAttnThreads);
-  KLLM_REQUIRE(window >= 0, "attn_generic: negative window");
+  KLLM_REQUIRE(vd > 0 && vd <= kMaxHeadDim, "attn_generic: value width %d is outside [1, %d]", vd, kMaxHeadDim);
+  KLLM_REQUIRE(window >= 0 && chunk >= 0, "attn_generic: negative window or chunk");
   KLLM_REQUIRE(H <= 65535, "attn_generic: too many heads for the grid");
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "attn_generic: unknown dtype %d", dtype);
   const dim3 grid(n, H);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kAttnThreads), 0, stream,
                        (const float*)q, (float*)out, (const float*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, hd, window, scale, slopes);
+                       block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes);
   else
     hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(kAttnThreads), 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions,
-                       span_of_token, block_table, max_pages, page_size, H, KV, hd, window, scale, slopes);
+                       span_of_token, block_table, max_pages, page_size, H, KV, hd, vd, window, chunk, sink, scale, slopes);
   KLLM_CHECK_LAUNCH("attn_generic");
   return 0;
 }

@@ -55,7 +55,36 @@ __device__ __forceinline__ float unary_act(float z, int act, float a_pos, float 
   return gate_act(z, act);
 }
 
+// The first key that the query at position `pos` reads: with a window the last `window`
+// positions, with a chunked mask nothing before the start of the query's own chunk of
+// `chunk` positions (chunks are counted from position 0); 0 switches either off.  Both
+// bounds grow with the position, which the kernels that take blocks of queries rely on.
+__host__ __device__ __forceinline__ int first_key(int pos, int window, int chunk) {
+  int start = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  if (chunk > 0) {
+    const int c = pos - pos % chunk;
+    start = c > start ? c : start;
+  }
+  return start;
+}
+
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.f / (1.f + expf(-v)); }
+
+// A gate and the sum it gates, for kernels that take both: act(g) * u for the gates' activations,
+// or the clamped gate: with g' = min(g, limit) and u' = clamp(u, -limit, limit),
+// g' sigmoid(alpha g') (u' + 1).
+enum : int { GATE_CLAMPED_SWISH = 4, GATED_COUNT = 5 };
+
+__host__ __device__ __forceinline__ bool gated_known(int act) { return (act >= 0 && act < ACT_COUNT) || act == GATE_CLAMPED_SWISH; }
+
+__device__ __forceinline__ float gated(float g, float u, int act, float limit, float alpha) {
+  if (act == GATE_CLAMPED_SWISH) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoid_f32(alpha * g) * (u + 1.f);
+  }
+  return gate_act(g, act) * u;
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

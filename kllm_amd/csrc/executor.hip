@@ -40,6 +40,14 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_delta_prep),
     KLLM_CMD_OP(kllm_delta_scan),
     KLLM_CMD_OP(kllm_delta_out),
+    KLLM_CMD_OP(kllm_norm_residual),
+    KLLM_CMD_OP(kllm_rope_tables_freq),
+    KLLM_CMD_OP(kllm_qkv_norm_append),
+    KLLM_CMD_OP(kllm_gate_bias),
+    KLLM_CMD_OP(kllm_moe_route),
+    KLLM_CMD_OP(kllm_moe_plan),
+    KLLM_CMD_OP(kllm_moe_expert),
+    KLLM_CMD_OP(kllm_moe_combine),
 };
 constexpr int kNumOps = (int)(sizeof(kOps) / sizeof(kOps[0]));
 

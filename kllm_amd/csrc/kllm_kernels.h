@@ -209,11 +209,14 @@ int kllm_fused_linear(const void* x, int x_stride, const KllmLinearOut* out, con
 /* Causal attention of n tokens over the paged cache; any head size up to 256.
  * `slopes` (here and in the other attention entry points; null: none) holds one number per
  * head: slopes[h] * (query position - key position) is taken off the scaled score, a bias
- * that grows with the distance to the key. */
+ * that grows with the distance to the key.
+ * `vd`: width of a value (a page holds keys [KV][slot][hd], then values [KV][vd][slot]);
+ * `chunk` > 0: the query at position p reads no key before p - p % chunk; `sink` != 0: the
+ * softmax's denominator has one more term, exp(0). */
 int kllm_attn_generic(const void* q, void* out, const void* cache, const int* positions,
                       const int* span_of_token, const int* block_table, int max_pages,
-                      int page_size, int n, int H, int KV, int hd, int window, float scale,
-                      const float* slopes, int dtype, hipStream_t stream);
+                      int page_size, int n, int H, int KV, int hd, int vd, int window, int chunk,
+                      int sink, float scale, const float* slopes, int dtype, hipStream_t stream);
 
 /* Decode attention on the matrix cores: every token's keys are cut into
  * `nslices` slices (1..256) that run side by side (bfloat16: a workgroup of 4
@@ -328,6 +331,53 @@ int kllm_delta_scan(const float* scan_in, float* o_out, float* state, const int*
                     hipStream_t stream);
 int kllm_delta_out(const float* o, const float* gate, const float* weight, float eps, void* out, int n, int H,
                    int hd, int dtype, hipStream_t stream);
+
+/* Layers whose norm stands behind the sub-layer.  x [n, d] float32.  With sums (`delta`, float32
+ * [nsplit][n][d], plus `bias` [d] or null): x += weight * N(delta + bias); without: x = weight *
+ * N(x); N(v) = v / sqrt(mean(v^2) + eps).  `out` (or null) receives the new rows of x in
+ * `out_dtype`, for the next product. */
+int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
+                       const float* weight, void* out, int out_dtype, int n, int d, float eps,
+                       hipStream_t stream);
+/* cos/sin [n][half] = factor * cos/sin(positions[t] * freq[i]), the angle in double. */
+int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, const double* freq, int n,
+                          int half, double factor, hipStream_t stream);
+/* qkv: float32 sums [nsplit][n][(H + KV) dk + KV dv] of the query, key and value products.  Adds
+ * `bias` (or null), turns the first `rot` elements of every query and key head (pairs (2j, 2j+1)
+ * if `interleaved`, else (j, j + rot/2); cos/sin [n][rot/2] or null), divides every query and
+ * key head by its root mean square (`unit_norm`, eps inside the root), writes the queries and
+ * appends keys and values to the pages (keys [KV][slot][dk], then values [KV][dv][slot]). */
+int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_stride, const float* bias,
+                         const float* cos_t, const float* sin_t, int rot, int interleaved, int unit_norm,
+                         float eps, void* q_out, void* cache, const int* positions,
+                         const int* span_of_token, const int* block_table, int max_pages, int page_size,
+                         int n, int H, int KV, int dk, int dv, int dtype, hipStream_t stream);
+/* out [n][f] = gated(g, u) of the float32 sums gu [nsplit][n][2 f] (gates, then ups) plus `bias`
+ * [2 f] or null.  act: a gate's activation (act(g) u), or 4: with g' = min(g, limit) and u' =
+ * clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1). */
+int kllm_gate_bias(const float* gu, int nsplit, long split_stride, const float* bias, void* out,
+                   int out_dtype, int n, int f, int act, float limit, float alpha, hipStream_t stream);
+
+/* A routed feed-forward.  route: z float32 sums [nsplit][n][R] of the router over all R experts;
+ * idx/wgt [n][top] receive the `top` experts with the largest softmax(z) + correction (null: none)
+ * and their softmax scores divided by their sum.  plan: the entries (token * top + choice) whose
+ * expert is below E, grouped by expert into `sorted`, and `tiles` [max_tiles][3] = (expert, first
+ * place in sorted, entries <= kllm_moe_tile_rows()); max_tiles >= ceil(entries / rows) + E.
+ * expert, mode 0: out [entries][m] (dtype) = gated(gate, up) of x [tokens][k] against w [E][2 m][k];
+ * mode 1: out [entries][m] float32 = x [entries][k] against w [E][m][k].  combine: out [n][d] =
+ * sum over a token's choices of wgt * (expert < E ? y [entries][d] : xin [n][d]) + the slices of
+ * `shared` [ns][n][d] (null: none). */
+int kllm_moe_tile_rows(void);
+int kllm_moe_route(const float* z, int nsplit, long split_stride, const float* correction, int n, int R,
+                   int top, int* idx, float* wgt, hipStream_t stream);
+int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int* sorted, int* tiles,
+                  hipStream_t stream);
+int kllm_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
+                    int max_tiles, int top, int m, int k, int mode, int act, float limit, float alpha,
+                    int dtype, hipStream_t stream);
+int kllm_moe_combine(const float* y, const void* xin, const int* idx, const float* wgt, const float* shared,
+                     int ns, long shared_stride, float* out, int n, int d, int top, int E, int dtype,
+                     hipStream_t stream);
 
 /* out[r] = sampled index of logits[r][:]; temperature/uniform null: greedy. */
 int kllm_sample(int* out, const float* logits, const float* temperature, const float* uniform,

@@ -1,0 +1,230 @@
+// Per-token steps of layers whose norm stands behind the sub-layer instead of in front of it,
+// and of attention whose queries and keys are normalised after their rotation:
+//
+//   kllm_norm_residual     x += w * N(d + b), or x = w * N(x); N(v) = v / sqrt(mean(v^2) + eps);
+//                          optionally x rounded to the compute dtype for the next product
+//   kllm_rope_tables_freq  cos/sin tables from a table of angles per position (any schedule of
+//                          frequencies), times a constant factor
+//   kllm_qkv_norm_append   biases, rotation of the leading elements of every head, unit RMS of
+//                          every query and key head, queries out, keys and values into pages
+//   kllm_gate_bias         the gate of a gated feed-forward whose two products have biases, or
+//                          whose gate is clamped
+//
+// Everything here is computed in 32-bit; a row's result depends on the row alone.
+#include <math.h>
+
+#include "common.hpp"
+#include "kllm_kernels.h"
+
+namespace kllm {
+
+constexpr int kRowThreads = 256;
+
+// One workgroup per row, the row's sums kept in LDS between the two passes.
+template <typename TOUT>
+__global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
+    float* __restrict__ x, const float* __restrict__ delta, int nsplit, long split_stride,
+    const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps) {
+  extern __shared__ float row_lds[];      // [d]
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float* xr = x + r * d;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += kRowThreads) {
+    float v;
+    if (delta) {
+      v = 0.f;
+      for (int s = 0; s < nsplit; ++s) v += delta[s * split_stride + r * d + i];
+      if (bias) v += bias[i];
+    } else {
+      v = xr[i];
+    }
+    row_lds[i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float total = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(total / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += kRowThreads) {    // a thread reads back what it wrote itself
+    const float y = row_lds[i] * rstd * w[i];
+    const float v = delta ? xr[i] + y : y;
+    xr[i] = v;
+    if (out) out[r * d + i] = from_f32<TOUT>(v);
+  }
+}
+
+__global__ void rope_tables_freq_kernel(float* __restrict__ cos_t, float* __restrict__ sin_t,
+                                        const int* __restrict__ positions, const double* __restrict__ freq, int n,
+                                        int half, double factor) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)n * half) return;
+  const int t = (int)(idx / half), i = (int)(idx % half);
+  double sn, cs;
+  sincos((double)positions[t] * freq[i], &sn, &cs);
+  cos_t[idx] = (float)(cs * factor);
+  sin_t[idx] = (float)(sn * factor);
+}
+
+// One wave per (token, item): the items of a token are its H query heads, its KV key heads and
+// its KV value heads.  A lane holds up to two pairs of a head of up to 256.
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_norm_append_kernel(
+    const float* __restrict__ qkv, int nsplit, long split_stride, const float* __restrict__ bias,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int interleaved, int unit_norm,
+    float eps, T* __restrict__ q_out, T* __restrict__ cache, const int* __restrict__ positions,
+    const int* __restrict__ span_of_token, const int* __restrict__ block_table, int max_pages, int page_size,
+    int H, int KV, int dk, int dv) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x % kWave;
+  const int item = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (item >= H + 2 * KV) return;
+  const long cols = (long)(H + KV) * dk + (long)KV * dv;
+  const float* in = qkv + t * cols;
+  const int pos = positions[t];
+  const long page = block_table[(long)span_of_token[t] * max_pages + pos / page_size];
+  const int slot = pos % page_size;
+  const long kblock = (long)page_size * dk, vblock = (long)page_size * dv;
+  T* page_base = cache + page * KV * (kblock + vblock);
+  auto sum_at = [&](long col) {
+    float v = 0.f;
+    for (int s = 0; s < nsplit; ++s) v += in[s * split_stride + col];
+    return bias ? v + bias[col] : v;
+  };
+  if (item >= H + KV) {     // a value head: stored with the slot as the fast index
+    const int h = item - H - KV;
+    T* vdst = page_base + KV * kblock + h * vblock + slot;
+    for (int j = lane; j < dv; j += kWave) vdst[(long)j * page_size] = from_f32<T>(sum_at((long)(H + KV) * dk + h * dv + j));
+    return;
+  }
+  const bool is_q = item < H;
+  const int h = is_q ? item : item - H;
+  const long base = (long)item * dk;         // queries first, then keys, head after head
+  const int pairs = dk / 2, rhalf = rot / 2;
+  float ra[2], rb[2];
+  int ea[2], eb[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int j = lane + kWave * r;
+    ra[r] = rb[r] = 0.f;
+    ea[r] = eb[r] = 0;
+    if (j >= pairs) continue;
+    const bool turns = cos_t && j < rhalf;
+    // the two elements of this pair: one that turns, or two neighbours that pass through
+    ea[r] = j < rhalf ? (interleaved ? 2 * j : j) : rot + 2 * (j - rhalf);
+    eb[r] = j < rhalf ? (interleaved ? 2 * j + 1 : j + rhalf) : ea[r] + 1;
+    const float a = sum_at(base + ea[r]), b = sum_at(base + eb[r]);
+    const float c = turns ? cos_t[t * rhalf + j] : 1.f, s = turns ? sin_t[t * rhalf + j] : 0.f;
+    ra[r] = a * c - b * s;
+    rb[r] = b * c + a * s;
+    ss += ra[r] * ra[r] + rb[r] * rb[r];
+  }
+  float rstd = 1.f;
+  if (unit_norm) rstd = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+  T* dst = is_q ? q_out + (t * H + h) * dk : page_base + h * kblock + (long)slot * dk;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    if (lane + kWave * r >= pairs) continue;
+    dst[ea[r]] = from_f32<T>(ra[r] * rstd);
+    dst[eb[r]] = from_f32<T>(rb[r] * rstd);
+  }
+}
+
+template <typename TOUT>
+__global__ void gate_bias_kernel(const float* __restrict__ gu, int nsplit, long split_stride,
+                                 const float* __restrict__ bias, TOUT* __restrict__ out, long count, int f, int act,
+                                 float limit, float alpha) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  const long t = idx / f;
+  const int j = (int)(idx % f);
+  const float* row = gu + t * 2 * f;
+  float g = 0.f, u = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    g += row[s * split_stride + j];
+    u += row[s * split_stride + f + j];
+  }
+  if (bias) {
+    g += bias[j];
+    u += bias[f + j];
+  }
+  out[idx] = from_f32<TOUT>(gated(g, u, act, limit, alpha));
+}
+
+}  // namespace kllm
+
+using namespace kllm;
+
+extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
+                                  const float* weight, void* out, int out_dtype, int n, int d, float eps,
+                                  hipStream_t stream) {
+  KLLM_REQUIRE(x && weight, "norm_residual: null pointer");
+  KLLM_REQUIRE(n > 0 && d > 0 && d <= 16384, "norm_residual: bad sizes n=%d d=%d (rows of up to 16384)", n, d);
+  KLLM_REQUIRE(!delta || nsplit >= 1, "norm_residual: nsplit %d", nsplit);
+  KLLM_REQUIRE(delta || !bias, "norm_residual: a bias goes with sums");
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "norm_residual: unknown dtype %d", out_dtype);
+  const size_t lds = (size_t)d * sizeof(float);
+  if (out && out_dtype == DT_BF16)
+    hipLaunchKernelGGL(norm_residual_kernel<bf16_t>, dim3(n), dim3(kRowThreads), lds, stream, x, delta, nsplit,
+                       split_stride, bias, weight, (bf16_t*)out, d, eps);
+  else
+    hipLaunchKernelGGL(norm_residual_kernel<float>, dim3(n), dim3(kRowThreads), lds, stream, x, delta, nsplit,
+                       split_stride, bias, weight, (float*)out, d, eps);
+  KLLM_CHECK_LAUNCH("norm_residual");
+  return 0;
+}
+
+extern "C" int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, const double* freq, int n,
+                                     int half, double factor, hipStream_t stream) {
+  KLLM_REQUIRE(cos_t && sin_t && positions && freq, "rope_tables_freq: null pointer");
+  KLLM_REQUIRE(n > 0 && half > 0, "rope_tables_freq: bad sizes n=%d half=%d", n, half);
+  hipLaunchKernelGGL(rope_tables_freq_kernel, dim3(ceil_div((long)n * half, 256)), dim3(256), 0, stream, cos_t, sin_t,
+                     positions, freq, n, half, factor);
+  KLLM_CHECK_LAUNCH("rope_tables_freq");
+  return 0;
+}
+
+extern "C" int kllm_qkv_norm_append(const float* qkv, int nsplit, long split_stride, const float* bias,
+                                    const float* cos_t, const float* sin_t, int rot, int interleaved, int unit_norm,
+                                    float eps, void* q_out, void* cache, const int* positions,
+                                    const int* span_of_token, const int* block_table, int max_pages, int page_size,
+                                    int n, int H, int KV, int dk, int dv, int dtype, hipStream_t stream) {
+  KLLM_REQUIRE(qkv && q_out && cache && positions && span_of_token && block_table, "qkv_norm_append: null pointer");
+  KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && nsplit >= 1, "qkv_norm_append: bad sizes n=%d H=%d KV=%d nsplit=%d", n, H, KV,
+               nsplit);
+  KLLM_REQUIRE(dk > 0 && dk % 2 == 0 && dk <= 256 && dv > 0 && dv <= 256,
+               "qkv_norm_append: heads of %d (even) and values of %d, up to 256", dk, dv);
+  KLLM_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0 && (interleaved == 0 || interleaved == 1),
+               "qkv_norm_append: rotary dimension %d of a head of %d", rot, dk);
+  KLLM_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "qkv_norm_append: cos and sin go together");
+  KLLM_REQUIRE(max_pages > 0 && page_size > 0, "qkv_norm_append: bad cache sizes");
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "qkv_norm_append: unknown dtype %d", dtype);
+  const dim3 grid(n, ceil_div(H + 2 * KV, 4));
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(qkv_norm_append_kernel<float>, grid, dim3(256), 0, stream, qkv, nsplit, split_stride, bias, cos_t,
+                       sin_t, rot, interleaved, unit_norm, eps, (float*)q_out, (float*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, H, KV, dk, dv);
+  else
+    hipLaunchKernelGGL(qkv_norm_append_kernel<bf16_t>, grid, dim3(256), 0, stream, qkv, nsplit, split_stride, bias, cos_t,
+                       sin_t, rot, interleaved, unit_norm, eps, (bf16_t*)q_out, (bf16_t*)cache, positions, span_of_token,
+                       block_table, max_pages, page_size, H, KV, dk, dv);
+  KLLM_CHECK_LAUNCH("qkv_norm_append");
+  return 0;
+}
+
+extern "C" int kllm_gate_bias(const float* gu, int nsplit, long split_stride, const float* bias, void* out,
+                              int out_dtype, int n, int f, int act, float limit, float alpha, hipStream_t stream) {
+  KLLM_REQUIRE(gu && out, "gate_bias: null pointer");
+  KLLM_REQUIRE(n > 0 && f > 0 && nsplit >= 1, "gate_bias: bad sizes n=%d f=%d nsplit=%d", n, f, nsplit);
+  KLLM_REQUIRE(gated_known(act), "gate_bias: unknown activation %d", act);
+  KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "gate_bias: unknown dtype %d", out_dtype);
+  const long count = (long)n * f;
+  const dim3 grid(ceil_div(count, 256));
+  if (out_dtype == DT_BF16)
+    hipLaunchKernelGGL(gate_bias_kernel<bf16_t>, grid, dim3(256), 0, stream, gu, nsplit, split_stride, bias,
+                       (bf16_t*)out, count, f, act, limit, alpha);
+  else
+    hipLaunchKernelGGL(gate_bias_kernel<float>, grid, dim3(256), 0, stream, gu, nsplit, split_stride, bias, (float*)out,
+                       count, f, act, limit, alpha);
+  KLLM_CHECK_LAUNCH("gate_bias");
+  return 0;
+}

@@ -21,7 +21,7 @@ import torch
 DT_F32, DT_BF16 = 0, 1
 GEMM_PLAIN, GEMM_TILED_F32, GEMM_MFMA_BF16, GEMM_SKINNY_BF16, GEMM_GEMV, GEMM_GEMV_LDS, GEMM_MFMA_F32 = 0, 1, 2, 3, 4, 5, 6
 GEMV_BEST_ROWS = 0         # rows up to which they beat the MFMA kernels in bfloat16: none (a step at 1.1B sizes, one token: 1.036 against 0.963 ms)
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 
 class KernelError(RuntimeError):
@@ -112,7 +112,16 @@ def _declare(lib):
         "kllm_command_nargs": [I],
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
-        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, P],
+        "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, P],
+        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P],
+        "kllm_rope_tables_freq": [P, P, P, P, I, I, D, P],
+        "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "kllm_gate_bias": [P, I, L, P, P, I, I, I, I, F, F, P],
+        "kllm_moe_tile_rows": [],
+        "kllm_moe_route": [P, I, L, P, I, I, I, P, P, P],
+        "kllm_moe_plan": [P, I, I, I, P, P, P],
+        "kllm_moe_expert": [P, P, P, P, P, I, I, I, I, I, I, F, F, I, P],
+        "kllm_moe_combine": [P, P, P, P, P, I, L, P, I, I, I, I, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
         "kllm_device_cus": [],
@@ -155,7 +164,9 @@ LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_ap
              "kllm_sum_splits", "kllm_gemm", "kllm_gemm_swiglu", "kllm_gemv_plain", "kllm_gemv_swiglu",
              "kllm_gemv_resid", "kllm_gemv_rope_append", "kllm_fused_linear", "kllm_attn_generic",
              "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_gemm_act", "kllm_add_sinusoid", "kllm_unary_act",
-             "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out")
+             "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out",
+             "kllm_norm_residual", "kllm_rope_tables_freq", "kllm_qkv_norm_append", "kllm_gate_bias", "kllm_moe_route",
+             "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_combine")
 DYNAMIC_ARGS = {"kllm_attn_prefill": (16, 17)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
@@ -1019,15 +1030,29 @@ def _slopes(slopes, n_heads, who):
     return _ptr(slopes, who + " slopes", torch.float32, True)
 
 
+def paged_cache_fits(cache, n_kv_heads, page_size, head_dim, value_dim):
+    """Whether ``cache`` is a pool of pages for keys of ``head_dim`` and values of ``value_dim``:
+    [pages, 2, KV, page_size * head_dim] where the two are equal, or flat pages of
+    KV * page_size * (head_dim + value_dim) elements (keys [KV][slot][head_dim], then values
+    [KV][value_dim][slot]: the same place for every element where the widths are equal)."""
+    if cache.dim() == 4:
+        return head_dim == value_dim and tuple(cache.shape[1:]) == (2, n_kv_heads, page_size * head_dim)
+    return cache.dim() == 2 and cache.shape[1] == n_kv_heads * page_size * (head_dim + value_dim)
+
+
 def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size, n_heads,
-                 n_kv_heads, head_dim, window, scale, slopes=None):
+                 n_kv_heads, head_dim, window, scale, slopes=None, value_dim=None, chunk=0, sink=False):
     """``slopes`` (here and in the other attention wrappers): float32 [heads] or None; slopes[h]
-    times the distance from the query to the key is taken off head h's scaled scores."""
+    times the distance from the query to the key is taken off head h's scaled scores.
+    ``value_dim``: width of a value (default: the key's); ``chunk`` > 0: the query at position p
+    reads no key before p - p % chunk; ``sink``: the softmax's denominator has one more term,
+    exp(0)."""
     n = q.shape[0]
-    if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape)
+    vd = head_dim if value_dim is None else int(value_dim)
+    if (tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != (n, n_heads * vd)
             or q.dtype != cache.dtype or out.dtype != q.dtype):
         raise KernelError("attn_generic: q/out shapes or dtypes do not fit")
-    if tuple(cache.shape[1:]) != (2, n_kv_heads, page_size * head_dim):
+    if not paged_cache_fits(cache, n_kv_heads, page_size, head_dim, vd):
         raise KernelError(f"attn_generic: cache {tuple(cache.shape)} does not fit")
     if positions.numel() < n or span_of_token.numel() < n:
         raise KernelError("attn_generic: index arrays are too short")
@@ -1035,8 +1060,8 @@ def attn_generic(q, out, cache, positions, span_of_token, block_table, page_size
         _ptr(positions, "attn positions", torch.int32),
         _ptr(span_of_token, "attn span_of_token", torch.int32),
         _ptr(block_table, "attn block_table", torch.int32), block_table.shape[1], page_size, n,
-        n_heads, n_kv_heads, head_dim, int(window), float(scale), _slopes(slopes, n_heads, "attn_generic"),
-        dtype_code(q.dtype), _stream())
+        n_heads, n_kv_heads, head_dim, vd, int(window), int(chunk), int(bool(sink)), float(scale),
+        _slopes(slopes, n_heads, "attn_generic"), dtype_code(q.dtype), _stream())
 
 
 GENERIC_MAX_PAGE_SIZE = 256     # pages of the kernel that takes every size
@@ -1319,3 +1344,135 @@ def delta_out(o, gate, weight, eps, out, heads, head_dim):
     _launch("kllm_delta_out", "delta_out", _ptr(o, "delta_out o", F32), _ptr(gate, "delta_out gate", F32),
             _ptr(weight, "delta_out weight", F32), float(eps), _ptr(out, "delta_out out"), n, heads, head_dim,
             dtype_code(out.dtype), _stream())
+
+
+# ----------------------------------------------------------------------------- norm behind the sub-layer, rotation then unit norm, routed experts
+
+def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
+    """x [n, d] float32 in place.  With ``delta`` (float32 [n, d] or [nsplit, n, d]; ``bias`` [d] is
+    added to it): x += weight * N(delta + bias); without: x = weight * N(x), where N divides a
+    row by sqrt(mean of its squares + eps).  ``out`` [n, d] receives the new x in its own dtype."""
+    n, d = x.shape
+    nsplit, stride = (1, 0) if delta is None else _splits(delta, n, d, "norm_residual")
+    if weight.numel() != d or (bias is not None and bias.numel() != d) or (out is not None and tuple(out.shape) != (n, d)):
+        raise KernelError("norm_residual: weight, bias or output does not fit")
+    F32 = torch.float32
+    _launch("kllm_norm_residual", "norm_residual", _ptr(x, "norm_residual x", F32),
+            _ptr(delta, "norm_residual delta", F32, True), nsplit, stride, _ptr(bias, "norm_residual bias", F32, True),
+            _ptr(weight, "norm_residual weight", F32), _ptr(out, "norm_residual out", None, True),
+            dtype_code(out.dtype) if out is not None else DT_F32, n, d, float(eps), _stream())
+
+
+def rope_tables_freq(cos, sin, positions, freq, factor=1.0):
+    """cos, sin [n, half] = factor * cos/sin(positions[t] * freq[i]); freq: float64 [half]."""
+    n, half = cos.shape
+    if tuple(sin.shape) != (n, half) or freq.numel() != half or positions.numel() < n:
+        raise KernelError("rope_tables_freq: table shapes do not fit")
+    _launch("kllm_rope_tables_freq", "rope_tables_freq", _ptr(cos, "rope cos", torch.float32),
+            _ptr(sin, "rope sin", torch.float32), _ptr(positions, "rope positions", torch.int32),
+            _ptr(freq, "rope freq", torch.float64), n, half, float(factor), _stream())
+
+
+def qkv_norm_append(qkv, q_out, cache, positions, span_of_token, block_table, page_size, n_heads, n_kv_heads,
+                    head_dim, value_dim, bias=None, cos=None, sin=None, rotary_dim=0, interleaved=True,
+                    unit_norm=True, eps=0.0):
+    """qkv: float32 sums [nsplit, n, (H + KV) * head_dim + KV * value_dim].  Adds ``bias``, rotates the
+    first ``rotary_dim`` elements of every query and key head (cos, sin [n, rotary_dim / 2]),
+    divides every query and key head by its root mean square (``unit_norm``), writes q_out and
+    appends keys and values to the pages."""
+    n = q_out.shape[0]
+    cols = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
+    nsplit, stride = _splits(qkv, n, cols, "qkv_norm_append")
+    if q_out.shape[1] != n_heads * head_dim or (bias is not None and bias.numel() != cols):
+        raise KernelError("qkv_norm_append: q_out or bias does not fit")
+    if not paged_cache_fits(cache, n_kv_heads, page_size, head_dim, value_dim) or cache.dtype != q_out.dtype:
+        raise KernelError(f"qkv_norm_append: cache {tuple(cache.shape)} {cache.dtype} does not fit")
+    if positions.numel() < n or span_of_token.numel() < n:
+        raise KernelError("qkv_norm_append: index arrays are too short")
+    rot = int(rotary_dim) if cos is not None else 0
+    if cos is not None and (tuple(cos.shape) != (n, rot // 2) or tuple(sin.shape) != tuple(cos.shape)):
+        raise KernelError("qkv_norm_append: cos/sin shapes do not fit")
+    F32 = torch.float32
+    _launch("kllm_qkv_norm_append", "qkv_norm_append", _ptr(qkv, "qkv_norm_append qkv", F32), nsplit, stride,
+            _ptr(bias, "qkv_norm_append bias", F32, True), _ptr(cos, "qkv_norm_append cos", F32, True),
+            _ptr(sin, "qkv_norm_append sin", F32, True), rot, int(bool(interleaved)), int(bool(unit_norm)), float(eps),
+            _ptr(q_out, "qkv_norm_append q_out"), _ptr(cache, "qkv_norm_append cache"),
+            _ptr(positions, "qkv_norm_append positions", torch.int32),
+            _ptr(span_of_token, "qkv_norm_append span_of_token", torch.int32),
+            _ptr(block_table, "qkv_norm_append block_table", torch.int32), block_table.shape[1], page_size, n,
+            n_heads, n_kv_heads, head_dim, value_dim, dtype_code(q_out.dtype), _stream())
+
+
+GATE_CLAMPED_SWISH = 4     # g' = min(g, limit), u' = clamp(u, -limit, limit): g' sigmoid(alpha g') (u' + 1)
+GATES = dict(ACTIVATIONS, clamped_swish=GATE_CLAMPED_SWISH)
+
+
+def gate_bias(gu, out, act=ACT_SILU, bias=None, limit=0.0, alpha=1.0):
+    """out [n, f] = gated(gu[:, :f] + bias[:f], gu[:, f:] + bias[f:]); gu float32 sums [nsplit, n, 2f]."""
+    n, f = out.shape
+    nsplit, stride = _splits(gu, n, 2 * f, "gate_bias")
+    if bias is not None and bias.numel() != 2 * f:
+        raise KernelError("gate_bias: bias does not fit")
+    _launch("kllm_gate_bias", "gate_bias", _ptr(gu, "gate_bias in", torch.float32), nsplit, stride,
+            _ptr(bias, "gate_bias bias", torch.float32, True), _ptr(out, "gate_bias out"), dtype_code(out.dtype), n, f,
+            int(act), float(limit), float(alpha), _stream())
+
+
+def moe_tile_rows() -> int:
+    return limit("moe_tile_rows")
+
+
+def moe_max_tiles(entries, experts) -> int:
+    """Tiles that always hold ``entries`` (token, choice) pairs of ``experts`` experts."""
+    return -(-entries // moe_tile_rows()) + experts
+
+
+def moe_route(z, correction, idx, wgt):
+    """z: float32 sums [nsplit, n, R] of the router; idx int32, wgt float32 [n, top]."""
+    n, top = idx.shape
+    R = z.shape[-1]
+    nsplit, stride = _splits(z, n, R, "moe_route")
+    if tuple(wgt.shape) != (n, top) or (correction is not None and correction.numel() != R):
+        raise KernelError("moe_route: outputs or correction do not fit")
+    _launch("kllm_moe_route", "moe_route", _ptr(z, "moe_route z", torch.float32), nsplit, stride,
+            _ptr(correction, "moe_route correction", torch.float32, True), n, R, top,
+            _ptr(idx, "moe_route idx", torch.int32), _ptr(wgt, "moe_route wgt", torch.float32), _stream())
+
+
+def moe_plan(idx, experts, sorted_entries, tiles):
+    entries = idx.numel()
+    if sorted_entries.numel() < entries or tiles.dim() != 2 or tiles.shape[1] != 3:
+        raise KernelError("moe_plan: outputs do not fit")
+    _launch("kllm_moe_plan", "moe_plan", _ptr(idx, "moe_plan idx", torch.int32), entries, int(experts), tiles.shape[0],
+            _ptr(sorted_entries, "moe_plan sorted", torch.int32), _ptr(tiles, "moe_plan tiles", torch.int32), _stream())
+
+
+def moe_expert(x, w, out, sorted_entries, tiles, top, mode, act=ACT_SILU, limit=0.0, alpha=1.0):
+    """mode 0: x [tokens, k], w [E, 2m, k] -> out [tokens * top, m] gated, in x's dtype;
+    mode 1: x [tokens * top, k], w [E, m, k] -> out [tokens * top, m] float32."""
+    k = x.shape[1]
+    m = out.shape[1]
+    if (w.dim() != 3 or w.shape[2] != k or w.shape[1] != (2 * m if mode == 0 else m) or w.dtype != x.dtype
+            or out.dtype != (x.dtype if mode == 0 else torch.float32)
+            or out.shape[0] != (x.shape[0] * top if mode == 0 else x.shape[0]) or sorted_entries.numel() < out.shape[0]):
+        raise KernelError(f"moe_expert: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    _launch("kllm_moe_expert", "moe_expert", _ptr(x, "moe_expert x"), _ptr(w, "moe_expert w"), _ptr(out, "moe_expert out"),
+            _ptr(sorted_entries, "moe_expert sorted", torch.int32), _ptr(tiles, "moe_expert tiles", torch.int32),
+            tiles.shape[0], int(top), m, k, int(mode), int(act), float(limit), float(alpha), dtype_code(x.dtype),
+            _stream())
+
+
+def moe_combine(y, xin, idx, wgt, out, experts, shared=None):
+    """out [n, d] float32 = sum over choices of wgt * (idx < experts ? y[token * top + choice] : xin[token])
+    + the slices of ``shared`` (float32 [n, d] or [ns, n, d])."""
+    n, d = out.shape
+    top = idx.shape[1]
+    ns, stride = (0, 0)
+    if shared is not None:
+        ns, stride = _splits(shared, n, d, "moe_combine")
+    if tuple(y.shape) != (n * top, d) or tuple(xin.shape) != (n, d) or tuple(wgt.shape) != (n, top):
+        raise KernelError("moe_combine: shapes do not fit")
+    _launch("kllm_moe_combine", "moe_combine", _ptr(y, "moe_combine y", torch.float32), _ptr(xin, "moe_combine x"),
+            _ptr(idx, "moe_combine idx", torch.int32), _ptr(wgt, "moe_combine wgt", torch.float32),
+            _ptr(shared, "moe_combine shared", torch.float32, True), ns, stride,
+            _ptr(out, "moe_combine out", torch.float32), n, d, top, int(experts), dtype_code(xin.dtype), _stream())

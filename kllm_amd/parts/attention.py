@@ -11,7 +11,11 @@ Parameters: ``hidden``, ``heads``, ``kv_heads``, ``head_dim``, ``window``
 reads keys and values that another run cached and has no k/v projections),
 ``scale`` (default 1/sqrt(head_dim)), ``distance_slope_bits`` (None: no bias; b:
 head h's scaled scores lose 2^(-b (h+1) / heads) times the distance from the
-query to the key).
+query to the key), ``chunk`` (0: none; c: a chunked mask, the query at position
+p reads no key before p - p % c, chunks counted from the request's position 0),
+``sink`` (False; True: the softmax's denominator has one more term, exp(0): a
+key whose score is 0 and that has no value), ``value_dim`` (width of a value;
+default: the key's).
 Tensors: ``<prefix>.{q,k,v,o}_proj.weight``.  The three input projections are
 kept as one matrix so that a step reads one weight for them.
 """
@@ -40,6 +44,7 @@ class CausalSelfAttention(Part):
     step_lists_key = "attention.spans"
     SHORT_SPAN = 4
     QUERY_BLOCK = K.PREFILL_QUERY_BLOCK
+    FAST_KERNELS_OFF = False
 
     def step_lists(self, starts, lens):
         short, blocks = [], []
@@ -63,6 +68,8 @@ class CausalSelfAttention(Part):
             for first in range(0, n, self.QUERY_BLOCK):
                 last = pos + min(first + self.QUERY_BLOCK, n)          # keys [0, last) are before the block's end
                 keys = min(last, self.window + self.QUERY_BLOCK) if self.window else last
+                if self.chunk:      # nothing before the chunk of the block's first query
+                    keys = min(keys, last - (pos + first) // self.chunk * self.chunk)
                 total += keys
                 longest = max(longest, keys)
         return {"keys_total": total, "keys_longest": longest}
@@ -74,7 +81,13 @@ class CausalSelfAttention(Part):
         self.kv_heads = int(self.param("kv_heads"))
         self.head_dim = int(self.param("head_dim"))
         self.window = int(self.param("window", 0) or 0)
-        self.step_values_key = f"attention.keys.window{self.window}"     # layers with the same window read alike
+        self.chunk = int(self.param("chunk", 0) or 0)
+        self.sink = bool(self.param("sink", False))
+        self.value_dim = int(self.param("value_dim", None) or self.head_dim)
+        if self.chunk < 0 or not 0 < self.value_dim <= 256:
+            raise ValueError(f"attention: chunk {self.chunk} or value_dim {self.value_dim} out of range")
+        # layers with the same window and chunk read alike
+        self.step_values_key = f"attention.keys.window{self.window}" + (f".chunk{self.chunk}" if self.chunk else "")
         self.own_kv = bool(self.param("own_kv", True))
         if self.heads % self.kv_heads:
             raise ValueError(f"attention: {self.heads} heads are not a multiple of {self.kv_heads} KV heads")
@@ -98,6 +111,7 @@ class CausalSelfAttention(Part):
         self.slopes = None          # float32 [heads] on the device once bound
         self.q_dim = self.heads * self.head_dim
         self.kv_dim = self.kv_heads * self.head_dim
+        self.out_dim = self.heads * self.value_dim
         self.w_in = None
         self.w_o = None
         self._tiled = {}
@@ -131,7 +145,8 @@ class CausalSelfAttention(Part):
         self._tiled["o"] = tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)
 
     def cache_need(self):
-        return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window)
+        return CacheNeed("paged", kv_heads=self.kv_heads, head_dim=self.head_dim, window=self.window,
+                         value_dim=self.value_dim if self.value_dim != self.head_dim else None)
 
     def flops(self, tokens, keys_read=0.0):
         # the projections, and per key read a score and a value product for every head
@@ -211,11 +226,13 @@ class CausalSelfAttention(Part):
             prompt_ok = self.head_dim in K.PREFILL_HEAD_DIMS
         else:
             fast = prompt_ok = K.attn_f32_fits(self.head_dim, cache.page_size)
-        fast = fast and mode != "generic"
+        # the kernels on the matrix cores take keys and values of one width
+        fast = fast and mode != "generic" and self.value_dim == self.head_dim and not self.FAST_KERNELS_OFF
+        fast = fast and not self.chunk and not self.sink
         if not fast:
             K.attn_generic(q, out, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table,
                            cache.page_size, self.heads, self.kv_heads, self.head_dim, self.window,
-                           self.scale, slopes=self.slopes)
+                           self.scale, slopes=self.slopes, value_dim=self.value_dim, chunk=self.chunk, sink=self.sink)
             return
         n = q.shape[0]
         short = ctx.lists.get("attention.spans.short")
@@ -332,5 +349,68 @@ class KeysAsValuesAttention(CausalSelfAttention):
                          q_weight=self.q_norm, k_weight=self.k_norm, eps=self.eps, temp_coef=self.temp_coef,
                          temp_every=self.temp_every)
         out = ctx.buf("attn.out", (n, self.q_dim), dtype)
+        self.attend(ctx, q, out, cache)
+        return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))
+
+
+@register_part("mixer", "attention_unit_qk")
+class UnitNormAttention(CausalSelfAttention):
+    """Attention whose queries and keys are rotated and then divided, head by head, by their root
+    mean square (an RMS norm without a weight): q = W_q h + b_q, k = W_k h + b_k, v = W_v h + b_v;
+    the first ``rotary_dim`` elements of every query and key head turn with the position (the
+    position part says how); q and k become q / sqrt(mean(q^2) + eps) per head; the score is
+    (q . k) * ``scale``; mask (``window``, ``chunk``), ``sink`` and the kernels are the base
+    class's; values may have a width of their own (``value_dim``); the output projection has no
+    bias.
+
+    Parameters beyond the base class's: ``eps``, ``bias`` (default True: q, k and v have one).
+    Tensors: ``<prefix>.{q,k,v,o}.weight``, ``.{q,k,v}.bias``."""
+    takes_normed = False
+    fills_sink = False
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        if not self.own_kv:
+            raise ValueError("attention_unit_qk: keeps its own keys and values")
+        self.eps = float(self.param("eps"))
+        self.has_bias = bool(self.param("bias", True))
+        self.v_dim = self.kv_heads * self.value_dim
+        self.bias = None
+
+    def weight_specs(self):
+        specs = [WeightSpec(self.tensor_name("q.weight"), (self.q_dim, self.hidden)),
+                 WeightSpec(self.tensor_name("k.weight"), (self.kv_dim, self.hidden)),
+                 WeightSpec(self.tensor_name("v.weight"), (self.v_dim, self.hidden)),
+                 WeightSpec(self.tensor_name("o.weight"), (self.hidden, self.out_dim))]
+        if self.has_bias:
+            specs += [WeightSpec(self.tensor_name("q.bias"), (self.q_dim,), "vector"),
+                      WeightSpec(self.tensor_name("k.bias"), (self.kv_dim,), "vector"),
+                      WeightSpec(self.tensor_name("v.bias"), (self.v_dim,), "vector")]
+        return specs
+
+    def bind(self, weights):
+        self._bind_slopes()
+        self.w_in = torch.cat([weights[self.tensor_name(t + ".weight")] for t in ("q", "k", "v")], dim=0).contiguous()
+        self.w_o = weights[self.tensor_name("o.weight")]
+        self.bias = (torch.cat([weights[self.tensor_name(t + ".bias")] for t in ("q", "k", "v")]).contiguous()
+                     if self.has_bias else None)
+        # second copies for decode batches, in the order that kernel reads them
+        self._tiled = {"in": tiled_copy(self.runtime, self.w_in, K.LINEAR_PARTS),
+                       "o": tiled_copy(self.runtime, self.w_o, K.LINEAR_PARTS)}
+
+    def forward(self, ctx, xn, cache):
+        n = xn.shape[0]
+        dtype = self.runtime.dtype
+        if not cache.write:
+            raise ValueError("attention_unit_qk: the run writes its own cache")
+        qkv = decode_linear(ctx, xn, self.w_in, "attn.qkv", self._tiled.get("in"))
+        q = ctx.buf("attn.q", (n, self.q_dim), dtype)
+        cos = sin = None
+        if self.position is not None and hasattr(self.position, "tables"):
+            cos, sin = self.position.tables(ctx)
+        K.qkv_norm_append(qkv, q, cache.pages, ctx.positions, ctx.span_of_token, cache.block_table, cache.page_size,
+                          self.heads, self.kv_heads, self.head_dim, self.value_dim, bias=self.bias, cos=cos, sin=sin,
+                          rotary_dim=self.rotary_dim, interleaved=self.interleaved, unit_norm=True, eps=self.eps)
+        out = ctx.buf("attn.out", (n, self.out_dim), dtype)
         self.attend(ctx, q, out, cache)
         return decode_linear(ctx, out, self.w_o, "attn.proj", self._tiled.get("o"))

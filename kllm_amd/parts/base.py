@@ -264,6 +264,24 @@ class StepContext:
         return (self.workspace or self.runtime.workspace).get(tag, shape, dtype)
 
 
+def stream_copy(ctx, x, fill=True):
+    """The rows of the float32 residual stream ``x`` in the compute dtype, for sub-layers that
+    read the stream itself: x where the compute dtype is float32; otherwise a buffer that
+    whoever last changed x filled in the same launch (``fill`` False: the caller is about to;
+    it hands the buffer to its kernel, or None where none is needed), or that is filled here."""
+    from .. import kernels as K
+    if ctx.runtime.dtype == torch.float32:
+        return x if fill else None
+    held = ctx.scratch.get("stream.copy")
+    if held is not None and held[0] is x:
+        return held[1]
+    xb = ctx.buf("x.copy", tuple(x.shape), ctx.runtime.dtype)
+    ctx.scratch["stream.copy"] = (x, xb)
+    if fill:
+        K.sum_splits(x.unsqueeze(0), xb)
+    return xb
+
+
 def call_part(part, fn, *args, **kwargs):
     """Call ``fn`` (a method of ``part``) so that its work reaches the stream in program order:
     as it is for a part that records its launches, otherwise with the recorded launches run

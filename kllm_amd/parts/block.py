@@ -12,7 +12,8 @@ norm's row scale to its own sums (``Normed``).
 
 from __future__ import annotations
 
-from .base import Part, ResidualSink, ScaledSum, call_part, make_part, register_part
+from .. import kernels as K
+from .base import Part, ResidualSink, ScaledSum, call_part, make_part, register_part, stream_copy
 
 
 @register_part("block", "pre_norm")
@@ -149,3 +150,72 @@ class ParallelBlock(Part):
         if self.feed_forward is not None:
             deltas.append(call_part(self.feed_forward, self.feed_forward.forward, ctx, xn))
         return x, ScaledSum(deltas, self.bias, self.mult)
+
+
+@register_part("block", "sublayer_norm")
+class SublayerNormBlock(Part):
+    """The norm stands behind each sub-layer, on its output alone, and the sub-layers read the
+    stream itself: a = x + Norm1(Mixer(x)); x' = a + Norm2(FeedForward(a)).  The layer may have
+    no feed-forward.  Both norms are RMS norms with ``weight`` and ``eps``; each is one launch
+    that adds the sums of the sub-layer's last product (and its bias, ``out_bias`` of a part),
+    normalises, adds to the float32 stream and leaves the stream's new rows in the compute
+    dtype for the next sub-layer.  Nothing stays pending behind the layer.
+
+    Parameters: ``layer``."""
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        layer = self.param("layer")
+        self.mixer = make_part("mixer", layer.mixer, runtime)
+        self.norm_mixer = make_part("norm", layer.norm_mixer, runtime)
+        self.feed_forward = (make_part("feed_forward", layer.feed_forward, runtime)
+                             if layer.feed_forward is not None else None)
+        self.norm_ff = make_part("norm", layer.norm_feed_forward, runtime) if self.feed_forward is not None else None
+        for norm in (self.norm_mixer, self.norm_ff):
+            if norm is not None and not (hasattr(norm, "weight") and hasattr(norm, "eps") and getattr(norm, "groups", 1) == 1):
+                raise ValueError("sublayer_norm: its norms are RMS norms with a weight and eps")
+
+    def parts(self):
+        return [p for p in (self.mixer, self.norm_mixer, self.feed_forward, self.norm_ff) if p is not None]
+
+    def children(self):
+        return self.parts()
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self.parts())
+
+    def weight_specs(self):
+        return [s for p in self.parts() for s in p.weight_specs()]
+
+    def bind(self, weights):
+        for p in self.parts():
+            p.bind(weights)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def read_bytes(self, tokens):
+        out = {}
+        for p in self.parts():
+            out.update(p.read_bytes(tokens))
+        return out
+
+    def flops(self, tokens, keys_read=0.0):
+        return sum(p.flops(tokens, keys_read) for p in self.parts())
+
+    def forward(self, ctx, x, pending, cache):
+        if pending is not None:
+            raise ValueError("sublayer_norm: the layer in front of it left sums pending, which it has no norm for")
+        xin = stream_copy(ctx, x)
+        delta = call_part(self.mixer, self.mixer.forward, ctx, xin, cache)
+        out = stream_copy(ctx, x, fill=False)
+        K.norm_residual(x, self.norm_mixer.weight, delta, bias=getattr(self.mixer, "out_bias", None), out=out,
+                        eps=self.norm_mixer.eps)
+        if self.feed_forward is not None:
+            xin = stream_copy(ctx, x)
+            delta = call_part(self.feed_forward, self.feed_forward.forward, ctx, xin)
+            K.norm_residual(x, self.norm_ff.weight, delta, bias=getattr(self.feed_forward, "out_bias", None), out=out,
+                            eps=self.norm_ff.eps)
+        return x, None

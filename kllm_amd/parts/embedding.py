@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from .. import kernels as K
-from .base import Part, register_part
+from .base import Part, register_part, stream_copy
 from .linear import linear, tiled_copy
 from .spec import WeightSpec
 
@@ -30,12 +30,21 @@ class TokenEmbedding(Part):
         # an encoding that acts on the embedded tokens (``on_embedding``): the model calls it
         pos = self.param("position", None)
         self.position = runtime.shared_part("position", pos) if pos is not None else None
+        # an RMS norm of the embedded tokens, ``norm_eps`` (None: none); tensor ``<prefix>.norm``
+        eps = self.param("norm_eps", None)
+        self.norm_eps = float(eps) if eps is not None else None
+        self.norm_weight = None
 
     def weight_specs(self):
-        return [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]
+        specs = [WeightSpec(self.tensor_name("weight"), (self.vocab, self.hidden))]
+        if self.norm_eps is not None:
+            specs.append(WeightSpec(self.tensor_name("norm"), (self.hidden,), "vector"))
+        return specs
 
     def bind(self, weights):
         self.table = weights[self.tensor_name("weight")]
+        if self.norm_eps is not None:
+            self.norm_weight = weights[self.tensor_name("norm")]
 
     def read_bytes(self, tokens):
         return {self.table.data_ptr(): tokens * self.hidden * self.table.element_size()}   # one row per token
@@ -49,6 +58,8 @@ class TokenEmbedding(Part):
             K.embed(x, self.table, token_ids, ctx.token_from, ctx.sampled)
         else:
             K.embed(x, self.table, token_ids)
+        if self.norm_eps is not None:
+            K.norm_residual(x, self.norm_weight, eps=self.norm_eps, out=stream_copy(ctx, x, fill=False))
         return x
 
 

@@ -147,3 +147,58 @@ class DenseFeedForward(Part):
             up = decode_linear(ctx, xn, self.w_up, "ffn.up", self._tiled.get("up"))
             K.unary_act(up, h, self.act, self.act_params)
         return decode_linear(ctx, h, self.w_down, "ffn.down", self._tiled.get("down"))
+
+
+def gated_hidden(ctx, xn, w_gu, intermediate, tag, tiled=None, bias=None, act=K.ACT_SILU, limit=0.0, alpha=1.0):
+    """h [n, intermediate] = gated(gate sums + bias, up sums + bias) in the compute dtype, for gates
+    that the products' own epilogues do not know (biases, the clamped gate): the product of
+    both, then one launch for the gate."""
+    n = xn.shape[0]
+    gu = decode_linear(ctx, xn, w_gu, tag + ".gu", tiled)
+    h = ctx.buf(tag + ".h", (n, intermediate), ctx.runtime.dtype)
+    K.gate_bias(gu, h, act, bias=bias, limit=limit, alpha=alpha)
+    return h
+
+
+@register_part("feed_forward", "gated_mlp_bias")
+class BiasedGatedFeedForward(Part):
+    """Gated feed-forward whose three projections have biases:
+    down(act(gate(x) + b_g) * (up(x) + b_u)) + b_d.  The down projection's bias is left to
+    whoever adds the output to the stream (``out_bias``).
+
+    Parameters: ``hidden``, ``intermediate``, ``activation`` (a gate's: "silu", "gelu_tanh").
+    Tensors: ``<prefix>.{gate,up,down}.weight`` and ``.bias``."""
+    graph_safe = True
+    records_launches = True
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.hidden = int(self.param("hidden"))
+        self.intermediate = int(self.param("intermediate"))
+        act = self.param("activation", "silu")
+        if act not in K.ACTIVATIONS:
+            raise ValueError(f"gated_mlp_bias: activation {act!r} is not built (one of {sorted(K.ACTIVATIONS)})")
+        self.act = K.ACTIVATIONS[act]
+        self.w_gu = self.w_down = self.bias_gu = self.out_bias = None
+        self._tiled = {}
+
+    def weight_specs(self):
+        f, d = self.intermediate, self.hidden
+        return [WeightSpec(self.tensor_name("gate.weight"), (f, d)), WeightSpec(self.tensor_name("up.weight"), (f, d)),
+                WeightSpec(self.tensor_name("down.weight"), (d, f)),
+                WeightSpec(self.tensor_name("gate.bias"), (f,), "vector"),
+                WeightSpec(self.tensor_name("up.bias"), (f,), "vector"),
+                WeightSpec(self.tensor_name("down.bias"), (d,), "vector")]
+
+    def bind(self, weights):
+        w = lambda n: weights[self.tensor_name(n)]
+        self.w_gu = torch.cat([w("gate.weight"), w("up.weight")], dim=0).contiguous()
+        self.bias_gu = torch.cat([w("gate.bias"), w("up.bias")]).contiguous()
+        self.w_down = w("down.weight")
+        self.out_bias = w("down.bias")
+        self._tiled = {"gu": tiled_copy(self.runtime, self.w_gu, K.LINEAR_PARTS),
+                       "down": tiled_copy(self.runtime, self.w_down, K.LINEAR_PARTS)}
+
+    def forward(self, ctx, xn):
+        h = gated_hidden(ctx, xn, self.w_gu, self.intermediate, "ffn", self._tiled.get("gu"), self.bias_gu, self.act)
+        return decode_linear(ctx, h, self.w_down, "ffn.down", self._tiled.get("down"))
