@@ -58,7 +58,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ final_out, float* __restrict__ part,
     const bf16_t* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ span_of_token,
-    const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window,
+    const int* __restrict__ block_table, int max_pages, int page_size, int H, int KV, int window, int chunk, int sink,
     float scale, const float* __restrict__ slopes, int head_tiles, const int* __restrict__ token_list) {
   constexpr int hd = 16 * HDT;
   constexpr int KS = (hd + 31) / 32;           // MFMA steps over head_dim for the scores
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
   const int slice = blockIdx.z * kDecodeWaves + wave;
 
   const int len = positions[t] + 1;
-  const int start = (window > 0 && len > window) ? len - window : 0;
+  const int start = first_key(len - 1, window, chunk);     // window and chunked mask
   const int first = start / 32 * 32;                       // tiles of 32 keys from here
   const int tiles = (len - first + 31) / 32;
   const int per = (tiles + nslices - 1) / nslices;
@@ -95,7 +95,10 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
                  : zero8;
   }
 
-  float m = -INFINITY, l = 0.f;
+  // A sink (a key whose score is 0 and that has no value) is where the running maximum and
+  // sum of the first slice start: one of the four lanes of a column holds its exp(0).
+  const bool owns_sink = sink && slice == 0;
+  float m = owns_sink ? 0.f : -INFINITY, l = (owns_sink && g == 0) ? 1.f : 0.f;
   floatx4 acc[HDT];
 #pragma unroll
   for (int i = 0; i < HDT; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void attn_decode_mfma_kernel(
 template <int HDT, int W>
 static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out, float* part,
                          const void* cache, const int* positions, const int* span_of_token,
-                         const int* block_table, int max_pages, int page_size, int H, int KV, int window,
+                         const int* block_table, int max_pages, int page_size, int H, int KV, int window, int chunk, int sink,
                          float scale, const float* slopes, int head_tiles, const int* token_list) {
   const int heads = H / KV < 16 ? H / KV : 16;
   const size_t lds = (size_t)W * heads * (16 * HDT + 4) * sizeof(float);
@@ -306,12 +309,12 @@ static int launch_decode(dim3 grid, hipStream_t stream, const void* q, void* out
     }
     hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W, true>), grid, dim3(64 * W), lds, stream,
                        (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
-                       block_table, max_pages, page_size, H, KV, window, scale, slopes, head_tiles, token_list);
+                       block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, head_tiles, token_list);
     return 0;
   }
   hipLaunchKernelGGL((attn_decode_mfma_kernel<HDT, W>), grid, dim3(64 * W), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, part, (const bf16_t*)cache, positions, span_of_token,
-                     block_table, max_pages, page_size, H, KV, window, scale, slopes, head_tiles, token_list);
+                     block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, head_tiles, token_list);
   return 0;
 }
 
@@ -408,21 +411,21 @@ extern "C" int kllm_attn_decode_slices(int n, int KV, int H, int hd, int dtype, 
 static int attn_decode_run(const char* who, const void* q, void* out, float* part, long part_floats,
                            const void* cache, const int* positions, const int* span_of_token,
                            const int* block_table, int max_pages, int page_size, int n, int H, int KV,
-                           int hd, int window, float scale, const float* slopes, int nslices, int dtype,
+                           int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, int dtype,
                            const int* token_list, int n_listed, hipStream_t stream) {
   KLLM_REQUIRE(q && out && part && cache && positions && span_of_token && block_table,
                "%s: null pointer", who);
   KLLM_REQUIRE(dtype == DT_BF16 || dtype == DT_F32, "%s: unknown dtype %d", who, dtype);
   KLLM_REQUIRE(n > 0 && H > 0 && KV > 0 && H % KV == 0, "%s: bad heads n=%d H=%d KV=%d", who, n, H, KV);
   if (dtype == DT_F32) {
-    KLLM_REQUIRE(max_pages > 0 && window >= 0, "%s: bad table width or window", who);
+    KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "%s: bad table width, window or chunk", who);
     KLLM_REQUIRE(nslices >= 1 && part_floats >= (long)n * H * nslices * (hd + 2),
                  "%s: the partial results of n=%d H=%d nslices=%d head_dim=%d need %ld floats, the workspace has %ld",
                  who, n, H, nslices, hd, (long)n * H * nslices * (hd + 2), part_floats);
     KLLM_REQUIRE(H <= 65535, "%s: too many heads for the grid", who);
     KLLM_REQUIRE(!token_list || (n_listed > 0 && n_listed <= n), "%s: bad token list", who);
     return attn_f32_decode((const float*)q, (float*)out, part, (const float*)cache, positions, span_of_token,
-                           block_table, max_pages, page_size, H, KV, hd, window, scale, slopes, nslices, token_list,
+                           block_table, max_pages, page_size, H, KV, hd, window, chunk, sink, scale, slopes, nslices, token_list,
                            token_list ? n_listed : n, stream);
   }
   KLLM_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
@@ -430,7 +433,7 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
   KLLM_REQUIRE(page_size % 16 == 0 && page_size > 0 && max_pages > 0,
                "%s: page_size %d must be a multiple of 16", who, page_size);
   KLLM_REQUIRE(nslices >= 1 && nslices <= 256, "%s: nslices %d is outside [1, 256]", who, nslices);
-  KLLM_REQUIRE(window >= 0, "%s: negative window", who);
+  KLLM_REQUIRE(window >= 0 && chunk >= 0, "%s: negative window or chunk", who);
   KLLM_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)cache & 15) == 0 &&
                    ((uintptr_t)part & 15) == 0,
                "%s: q, out, cache and part must be 16-byte aligned", who);
@@ -447,11 +450,11 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
     if (int rc = nslices == 1                                                                     \
                      ? launch_decode<HDT, decode_waves_whole(HDT)>(                               \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, scale, slopes,          \
+                           block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes,          \
                            head_tiles, token_list)                                                            \
                      : launch_decode<HDT, kDecodeWavesShared>(                                    \
                            grid, stream, q, out, part, cache, positions, span_of_token,           \
-                           block_table, max_pages, page_size, H, KV, window, scale, slopes,          \
+                           block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes,          \
                            head_tiles, token_list))                                                           \
       return rc;                                                                                  \
     break
@@ -471,10 +474,10 @@ static int attn_decode_run(const char* who, const void* q, void* out, float* par
 extern "C" int kllm_attn_decode(const void* q, void* out, float* part, long part_floats,
                                 const void* cache, const int* positions, const int* span_of_token,
                                 const int* block_table, int max_pages, int page_size, int n, int H,
-                                int KV, int hd, int window, float scale, const float* slopes, int nslices, int dtype,
+                                int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, int dtype,
                                 const int* token_list, int n_listed, hipStream_t stream) {
   return attn_decode_run("attn_decode", q, out, part, part_floats, cache, positions, span_of_token,
-                         block_table, max_pages, page_size, n, H, KV, hd, window, scale, slopes, nslices, dtype,
+                         block_table, max_pages, page_size, n, H, KV, hd, window, chunk, sink, scale, slopes, nslices, dtype,
                          token_list, n_listed, stream);
 }
 
@@ -541,6 +544,6 @@ extern "C" int kllm_attn_decode_static(const void* q, void* out, const void* cac
   // Nothing in the scratch has to start at zero: the first kernel writes every partial result
   // (maximum, sum, output of each token, head and slice) that the second one reads.
   return attn_decode_run("attn_decode_static", q, out, part, (long)KLLM_ATTN_DECODE_STATIC_FLOATS, cache,
-                         positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window,
+                         positions, span_of_token, block_table, max_pages, page_size, n, H, KV, hd, window, 0, 0,
                          scale, nullptr, nslices, dtype, token_list, n_listed, stream);
 }

@@ -60,6 +60,7 @@ struct AttnF32Args {
   const int* block_table;
   int count;                   // decode: tokens; prompt: blocks of 128
   int max_pages, page_size, H, KV, hd, window;
+  int chunk, sink;             // a chunked mask (0: none); a key whose score is 0 and that has no value
   float scale;
   const float* slopes;         // per head: a bias that grows with the distance to the key (null: none)
   int nslices, col_blocks;     // decode: slices of the keys, blocks of 32 heads per group
@@ -145,10 +146,10 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
   const int my_tok = DECODE ? t_base : t_base + cc;
   const int my_head = DECODE ? h_base + cc : h_base;
   const int my_pos = DECODE ? pos_base : pos_base + cc;
-  const int my_start = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const int my_start = first_key(my_pos, window, a.chunk);
   const float my_slope = a.slopes ? a.slopes[my_head] : 0.f;
   const int qmax = DECODE ? pos_base : pos_base + ncol - 1;            // last key any column reads
-  const int lowest = window > 0 ? max(0, pos_base - window + 1) : 0;   // first key any column reads
+  const int lowest = first_key(pos_base, window, a.chunk);             // first key any column reads
   const int first = lowest / 32 * 32;
   const int tiles = (qmax - first) / 32 + 1;
   const int nslices = DECODE ? a.nslices : 1;
@@ -166,7 +167,10 @@ __global__ __launch_bounds__(64 * kF32Waves) void attn_f32_mfma_kernel(const Att
   const float* vcache = a.cache + ((long)KV + kvh) * block;
   const long page_stride = 2L * KV * block;
 
-  float m = -INFINITY, l = 0.f;
+  // A sink is where the running maximum and sum of the first slice start; one of a column's
+  // two lanes holds its exp(0).
+  const bool owns_sink = a.sink && slice == 0;
+  float m = owns_sink ? 0.f : -INFINITY, l = (owns_sink && g == 0) ? 1.f : 0.f;
   floatx16 acc[HDT];
 #pragma unroll
   for (int r = 0; r < HDT; ++r)
@@ -429,7 +433,7 @@ int attn_f32_slices(int n, int KV, int H, int max_keys) {
 
 int attn_f32_decode(const float* q, float* out, float* part, const float* cache, const int* positions,
                     const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                    int H, int KV, int hd, int window, float scale, const float* slopes, int nslices, const int* token_list,
+                    int H, int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, const int* token_list,
                     int count, hipStream_t stream) {
   KLLM_REQUIRE(attn_f32_fits(hd, page_size),
                "attn_decode float32: head_dim %d must be a multiple of 8 up to 256 and page_size %d a multiple of 4",
@@ -440,7 +444,7 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
   a.q = q; a.out = out; a.part = part; a.cache = cache;
   a.positions = positions; a.span_of_token = span_of_token; a.token_list = token_list;
   a.block_table = block_table; a.count = count;
-  a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window;
+  a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window; a.chunk = chunk; a.sink = sink;
   a.scale = scale; a.slopes = slopes; a.nslices = nslices; a.col_blocks = (H / KV + 31) / 32;
   a.wg_merge = nslices % kF32Waves == 0;
   const long items = (long)count * KV * a.col_blocks * nslices;
@@ -455,7 +459,7 @@ int attn_f32_decode(const float* q, float* out, float* part, const float* cache,
 
 int attn_f32_prefill(const float* q, float* out, const float* cache, const int* query_tiles, int n_tiles,
                      const int* span_start, const int* span_pos, const int* block_table, int max_pages,
-                     int page_size, int H, int KV, int hd, int window, float scale, const float* slopes, hipStream_t stream) {
+                     int page_size, int H, int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, hipStream_t stream) {
   KLLM_REQUIRE(attn_f32_fits(hd, page_size),
                "attn_prefill float32: head_dim %d must be a multiple of 8 up to 256 and page_size %d a multiple of 4",
                hd, page_size);
@@ -463,7 +467,7 @@ int attn_f32_prefill(const float* q, float* out, const float* cache, const int* 
   a.q = q; a.out = out; a.cache = cache;
   a.query_tiles = query_tiles; a.span_start = span_start; a.span_pos = span_pos;
   a.block_table = block_table; a.count = n_tiles;
-  a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window;
+  a.max_pages = max_pages; a.page_size = page_size; a.H = H; a.KV = KV; a.hd = hd; a.window = window; a.chunk = chunk; a.sink = sink;
   a.scale = scale; a.slopes = slopes; a.nslices = 1; a.col_blocks = 1;
   const long items = (long)n_tiles * 4 * H;
   if (int rc = dispatch_f32<false>(a, items, stream)) return rc;

@@ -18,14 +18,14 @@ bool attn_f32_fits(int hd, int page_size);
 // when nslices > 1.  Returns 0 or an error code (text set).
 int attn_f32_decode(const float* q, float* out, float* part, const float* cache, const int* positions,
                     const int* span_of_token, const int* block_table, int max_pages, int page_size,
-                    int H, int KV, int hd, int window, float scale, const float* slopes, int nslices, const int* token_list,
+                    int H, int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, int nslices, const int* token_list,
                     int count, hipStream_t stream);
 
 // Prompt tokens: query_tiles lists (first token row, span) of blocks of up to 128
 // consecutive tokens of one span; one wave per (32 tokens of a block, head).
 int attn_f32_prefill(const float* q, float* out, const float* cache, const int* query_tiles, int n_tiles,
                      const int* span_start, const int* span_pos, const int* block_table, int max_pages,
-                     int page_size, int H, int KV, int hd, int window, float scale, const float* slopes, hipStream_t stream);
+                     int page_size, int H, int KV, int hd, int window, int chunk, int sink, float scale, const float* slopes, hipStream_t stream);
 
 // Slices proposed for a decode batch of n tokens whose longest request has at most max_keys
 // keys (0: unknown).

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, unsigned page_magic, int H, int KV, int window, float scale, const float* __restrict__ slopes, float* __restrict__ part) {
+    int page_size, unsigned page_magic, int H, int KV, int window, int chunk, int sink, float scale, const float* __restrict__ slopes, float* __restrict__ part) {
   typedef PrefillShape<HDT> S;
   constexpr int hd = S::hd, KS = S::KS, NB = S::NB, KT = S::KT, KLD = S::KLD, VLD = S::VLD, CPT = S::CPT;
   extern __shared__ __attribute__((aligned(16))) bf16_t tiles_lds[];   // [PAR][2][kBuf]
@@ -110,9 +110,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const int tq = active ? wq0 + min(c, nq - 1) : t0;        // this lane's query (clamped)
   const int qpos = pos0 + (tq - s_begin);
   const int w_qmin = pos0 + (wq0 - s_begin), w_qmax = w_qmin + nq - 1;
-  const int lowest = (window > 0) ? max(0, blk_qmin - window + 1) : 0;   // first key any query reads
-  const int w_lowest = (window > 0) ? max(0, w_qmin - window + 1) : 0;   // ... any query of this wave
-  const int my_start = (window > 0) ? max(0, qpos - window + 1) : 0;
+  // (window and chunked mask: the first key a query reads does not fall as its position grows)
+  const int lowest = first_key(blk_qmin, window, chunk);      // first key any query reads
+  const int w_lowest = first_key(w_qmin, window, chunk);      // ... any query of this wave
+  const int my_start = first_key(qpos, window, chunk);
   const int* table = block_table + (long)span * max_pages;
   const long block = (long)page_size * hd;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -252,6 +253,11 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
   const float grow_raw = kGrow / c2;                        // kGrow in units of raw scores
   float mc = 0.f;                                           // m * c2, 0 while m is -inf
   float m_limit = -INFINITY;                                // m + grow_raw
+  if (sink && par == 0 && slice == 0) {   // a key whose score is 0 and that has no value: where one group's maximum and sum start
+    m = 0.f;
+    l = 1.f;
+    m_limit = grow_raw;
+  }
   auto tile_math = [&](auto masked, int kb, const bf16_t* buf) {
     // ---- scores: this lane's key rows are kb + c and kb + 32 + c
     floatx16 s[NB];
@@ -348,7 +354,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves * PAR) __attribute__((amdgpu_wav
     }
     l += ls[0];                                               // every row of ls is the sum over the tile's keys
   };
-  const int w_highstart = (window > 0) ? max(0, w_qmax - window + 1) : 0;   // from here on no query of the wave masks a key below it
+  const int w_highstart = first_key(w_qmax, window, chunk);   // from here on no query of the wave masks a key below it
   auto compute = [&](int t, const bf16_t* buf) {
     const int kb = tile_key(t);
     if (!active || kb > w_qmax || kb + KT <= w_lowest) return;   // nothing here for this wave's queries
@@ -483,7 +489,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
     const int* __restrict__ query_tiles, int n_tiles, const int* __restrict__ span_start,
     const int* __restrict__ span_pos, const int* __restrict__ block_table, int max_pages,
-    int page_size, int H, int KV, int window, float scale, const float* __restrict__ slopes) {
+    int page_size, int H, int KV, int window, int chunk, int sink, float scale, const float* __restrict__ slopes) {
   constexpr int hd = 32 * HDT;
   constexpr int KS = hd / 16;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -506,8 +512,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
   const int tq = t0 + min(c, nq - 1);                       // this lane's query (clamped)
   const int qpos = pos0 + (tq - s_begin);
   const int qpos_min = pos0 + (t0 - s_begin), qpos_max = qpos_min + nq - 1;
-  const int lowest = (window > 0) ? max(0, qpos_min - window + 1) : 0;   // first key any query reads
-  const int my_start = (window > 0) ? max(0, qpos - window + 1) : 0;
+  const int lowest = first_key(qpos_min, window, chunk);      // first key any query reads
+  const int my_start = first_key(qpos, window, chunk);
   const int* table = block_table + (long)span * max_pages;
   const long block = (long)page_size * hd;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -594,6 +600,11 @@ __global__ __launch_bounds__(64 * kPrefillWaves) __attribute__((amdgpu_waves_per
   const float grow_raw = kGrow / c2;                        // kGrow in units of raw scores
   float mc = 0.f;                                           // m * c2, 0 while m is -inf
   float m_limit = -INFINITY;                                // m + grow_raw
+  if (sink && wave == 0) {                // a key whose score is 0 and that has no value: where one wave's maximum and sum start
+    m = 0.f;
+    l = 1.f;
+    m_limit = grow_raw;
+  }
   auto compute = [&](const Tile& cur, int kb) {
     // ---- scores: this lane's key row is kb + c
     floatx16 s;
@@ -744,7 +755,7 @@ template <int HDT, int PAR>
 static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                                const int* query_tiles, int n_tiles, const int* span_start,
                                const int* span_pos, const int* block_table, int max_pages, int page_size,
-                               int H, int KV, int window, float scale, const float* slopes, float* part = nullptr, int nslices = 1) {
+                               int H, int KV, int window, int chunk, int sink, float scale, const float* slopes, float* part = nullptr, int nslices = 1) {
   typedef PrefillShape<HDT> S;
   const size_t lds = (size_t)PAR * 2 * S::kBuf * sizeof(bf16_t);   // also holds the groups' merge
   static int raised = 0;
@@ -756,7 +767,7 @@ static void launch_prefill_par(int grid, hipStream_t stream, const void* q, void
   const unsigned page_magic = (unsigned)(((1UL << 35) + page_size - 1) / page_size);   // ceil(2^35 / page_size)
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<HDT, PAR>), dim3(grid, nslices), dim3(64 * kPrefillWaves * PAR), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, scale, slopes, part);
+                     span_start, span_pos, block_table, max_pages, page_size, page_magic, H, KV, window, chunk, sink, scale, slopes, part);
   if (nslices > 1) {
     const dim3 mgrid(n_tiles * kQueryBlock, ceil_div(H, kMergeWaves));
     hipLaunchKernelGGL((attn_prefill_merge_kernel<(HDT + 1) / 2>), mgrid, dim3(64 * kMergeWaves), 0, stream,
@@ -768,7 +779,7 @@ template <int HDT>
 static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q, void* out, const void* cache,
                                  const int* query_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int window, float scale, const float* slopes) {
+                                 int window, int chunk, int sink, float scale, const float* slopes) {
   const size_t lds = (size_t)(kPrefillWaves - 1) * (HDT * 16 + 2) * kWave * sizeof(float);
   static int raised = 0;
   if (lds > 64 * 1024 && !raised) {
@@ -779,7 +790,7 @@ static void launch_prefill_split(int n_tiles, hipStream_t stream, const void* q,
   const int grid = n_tiles * (kQueryBlock / kQueryTile) * H;
   hipLaunchKernelGGL(attn_prefill_split_kernel<HDT>, dim3(grid), dim3(64 * kPrefillWaves), lds, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, query_tiles, n_tiles,
-                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, scale, slopes);
+                     span_start, span_pos, block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes);
 }
 
 // Which kernel.  One group of waves with the keys through LDS (three workgroups a CU) when
@@ -803,7 +814,7 @@ template <int HDT>
 static void launch_prefill(int grid, hipStream_t stream, const void* q, void* out, const void* cache,
                            const int* query_tiles, int n_tiles, const int* span_start,
                            const int* span_pos, const int* block_table, int max_pages, int page_size,
-                           int H, int KV, int window, float scale, const float* slopes, long keys_total,
+                           int H, int KV, int window, int chunk, int sink, float scale, const float* slopes, long keys_total,
                            int keys_longest, float* part, int nslices) {
   const int cus = device_cus();
   // (the caller asked kllm_attn_prefill_slices: few blocks of a large head.  The slices' results
@@ -811,7 +822,7 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
   // from about 1,280 keys to the longest block on, see there.)
   if (nslices > 1 && keys_longest >= kPrefillSliceFromKeys) {
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start,
-                                                        span_pos, block_table, max_pages, page_size, H, KV, window,
+                                                        span_pos, block_table, max_pages, page_size, H, KV, window, chunk, sink,
                                                         scale, slopes, part, nslices);
     return;
   }
@@ -820,14 +831,14 @@ static void launch_prefill(int grid, hipStream_t stream, const void* q, void* ou
     chain_bound = 5 * (keys_total * H / cus) < 6 * (long)keys_longest;
   if (grid > 2 * cus || PrefillShape<HDT>::kMaxPar == 1 || (grid > cus && !chain_bound))
     launch_prefill_par<HDT, 1>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,
-                               block_table, max_pages, page_size, H, KV, window, scale, slopes);
+                               block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes);
   else if (HDT >= 4 || 4 * grid > 3 * cus)
     launch_prefill_par<HDT, PrefillShape<HDT>::kMaxPar>(grid, stream, q, out, cache, query_tiles, n_tiles,
                                                         span_start, span_pos, block_table, max_pages, page_size,
-                                                        H, KV, window, scale, slopes);
+                                                        H, KV, window, chunk, sink, scale, slopes);
   else
     launch_prefill_split<HDT>(n_tiles, stream, q, out, cache, query_tiles, span_start, span_pos, block_table,
-                              max_pages, page_size, H, KV, window, scale, slopes);
+                              max_pages, page_size, H, KV, window, chunk, sink, scale, slopes);
 }
 
 }  // namespace kllm
@@ -853,7 +864,7 @@ extern "C" int kllm_attn_prefill_slices(int n_tiles, int H, int hd) {
 extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, const int* query_tiles,
                                  int n_tiles, const int* span_start, const int* span_pos,
                                  const int* block_table, int max_pages, int page_size, int H, int KV,
-                                 int hd, int window, float scale, const float* slopes, long keys_total, int keys_longest,
+                                 int hd, int window, int chunk, int sink, float scale, const float* slopes, long keys_total, int keys_longest,
                                  float* part, long part_floats, int nslices, int n_rows, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(q && out && cache && query_tiles && span_start && span_pos && block_table,
                "attn_prefill: null pointer");
@@ -862,15 +873,15 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
   KLLM_REQUIRE(n_tiles > 0 && H > 0 && KV > 0 && H % KV == 0, "attn_prefill: bad sizes tiles=%d H=%d KV=%d",
                n_tiles, H, KV);
   if (dtype == DT_F32) {
-    KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
+    KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "attn_prefill: bad table width, window or chunk");
     return attn_f32_prefill((const float*)q, (float*)out, (const float*)cache, query_tiles, n_tiles, span_start,
-                            span_pos, block_table, max_pages, page_size, H, KV, hd, window, scale, slopes, stream);
+                            span_pos, block_table, max_pages, page_size, H, KV, hd, window, chunk, sink, scale, slopes, stream);
   }
   KLLM_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256 && (hd <= 128 || hd == 192 || hd == 256),
                "attn_prefill: head_dim %d is not built (32, 64, 96, 128, 192, 256)", hd);
   KLLM_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_prefill: page_size %d must be a multiple of 16",
                page_size);
-  KLLM_REQUIRE(max_pages > 0 && window >= 0, "attn_prefill: bad table width or window");
+  KLLM_REQUIRE(max_pages > 0 && window >= 0 && chunk >= 0, "attn_prefill: bad table width, window or chunk");
   KLLM_REQUIRE(page_size <= kPrefillMaxPage && (long)max_pages * page_size <= kPrefillMaxKeys,
                "attn_prefill: page_size %d x table width %d beyond %d tokens per page or %d per request", page_size,
                max_pages, kPrefillMaxPage, kPrefillMaxKeys);
@@ -886,7 +897,7 @@ extern "C" int kllm_attn_prefill(const void* q, void* out, const void* cache, co
 #define KLLM_PF(HDT)                                                                              \
   case HDT:                                                                                       \
     launch_prefill<HDT>(grid, stream, q, out, cache, query_tiles, n_tiles, span_start, span_pos,  \
-                        block_table, max_pages, page_size, H, KV, window, scale, slopes, keys_total, \
+                        block_table, max_pages, page_size, H, KV, window, chunk, sink, scale, slopes, keys_total, \
                         keys_longest, part, nslices);                                             \
     break
   switch (hd / 32) {

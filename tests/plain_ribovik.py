@@ -76,6 +76,21 @@ def softmax_with_sink(s):
     return e / (torch.exp(-m) + e.sum(-1, keepdim=True))
 
 
+def masked_attention(q, k, v, scale, chunk, positions):
+    """q [n, H, d], k [n, G, d], v [n, G, dv] of one sequence at ``positions``: softmax with a sink
+    of the scaled scores of the keys a query reads, times the values; [n, H, dv]."""
+    n, H, _ = q.shape
+    G = k.shape[1]
+    mask = torch.tensor([[visible(i, j, chunk) for j in positions] for i in positions])
+    out = torch.zeros(n, H, v.shape[2], dtype=F64)
+    for hd in range(H):
+        g = hd // (H // G)
+        s = (q[:, hd] @ k[:, g].T) * float(scale)
+        s = s.masked_fill(~mask, float("-inf"))
+        out[:, hd] = softmax_with_sink(s) @ v[:, g]
+    return out
+
+
 def attention(h, w, p, m, eps, positions):
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     n = h.shape[0]
@@ -85,13 +100,7 @@ def attention(h, w, p, m, eps, positions):
     q = rms(rotate_neighbours(q, positions, m.get("rot")), eps)
     k = rms(rotate_neighbours(k, positions, m.get("rot")), eps)
     chunk = int((m.get("mask") or {}).get("size", 0))
-    mask = torch.tensor([[visible(i, j, chunk) for j in positions] for i in positions])
-    out = torch.zeros(n, H, dv, dtype=F64)
-    for hd in range(H):
-        g = hd // (H // G)
-        s = (q[:, hd] @ k[:, g].T) * float(m["scale"])
-        s = s.masked_fill(~mask, float("-inf"))
-        out[:, hd] = softmax_with_sink(s) @ v[:, g]
+    out = masked_attention(q, k, v, m["scale"], chunk, positions)
     return out.reshape(n, H * dv) @ w[p + ".o"].T
 
 
@@ -185,3 +194,36 @@ def tensor_shapes(cfg):
             if mlp.get("shared"):
                 three(p + ".shared", mlp["shared"]["ff"], False)
     return out
+
+
+def random_weights(cfg, seed, spaced_correction=False):
+    """Random float32 tensors of a checkpoint.  ``spaced_correction``: the corrections of a
+    router lie 1.5 apart in a shuffled order, more than two scores can differ, so that which
+    experts are chosen does not rest on small differences of the scores (the weights of the
+    chosen still do): for comparisons in bfloat16, where a close call falls either way."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        if name.endswith(".correction"):
+            n = shape[0]
+            if spaced_correction:
+                out[name] = 1.5 * torch.randperm(n, generator=g).float() - 0.75 * n
+            else:
+                out[name] = 0.05 * torch.randn(n, generator=g)
+        elif len(shape) == 1:
+            norm = "norm" in name.rsplit(".", 1)[-1] or name.endswith("norm")
+            out[name] = (1.0 + 0.2 * torch.randn(shape, generator=g)) if norm else 0.3 * torch.randn(shape, generator=g)
+        elif name == "embed":
+            out[name] = torch.randn(shape, generator=g)
+        elif name.endswith(".router"):
+            out[name] = 2.0 * torch.randn(shape, generator=g) / math.sqrt(shape[1])
+        else:
+            out[name] = 1.5 * torch.randn(shape, generator=g) / math.sqrt(shape[1])
+    return out
+
+
+def greedy(cfg, w, prompt, steps):
+    ids = list(prompt)
+    for _ in range(steps):
+        ids.append(int(forward(cfg, w, ids)[-1].argmax()))
+    return ids[len(prompt):]
