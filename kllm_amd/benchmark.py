@@ -339,15 +339,61 @@ def llama_config(width, heads, kv_heads, head_dim, ff, layers, vocab) -> dict:
             "rms_norm_eps": 1e-5, "tie_word_embeddings": False, "hidden_act": "silu"}
 
 
+# Ribovik beside Llama: the same attention sizes; the first layer's feed-forward is dense and as
+# wide as Llama's, the others are mixtures whose chosen experts and shared expert together are
+# about three quarters as wide.  The chunk of the mask is at least the context, so that both
+# models read as many keys.
+RIBOVIK_EXPERTS = {
+    "1.1b-sizes": dict(experts=16, identity=2, top=2, expert_ff=1408, shared_ff=1408),
+    "8b-sizes": dict(experts=8, identity=2, top=2, expert_ff=3584, shared_ff=3584),
+}
+
+
+def ribovik_config(width, heads, kv_heads, head_dim, ff, layers, vocab, experts=16, identity=2, top=2, expert_ff=1408,
+                   shared_ff=1408, chunk=4096) -> dict:
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+             "mask": {"size": chunk},
+             "rot": {"base": 500000.0, "dims": head_dim,
+                     "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0},
+           "router": {"experts": experts, "identity": identity, "top": top}, "shared": {"ff": shared_ff, "limit": 7.0}}
+    entries = [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if i == 0 else moe}
+               for i in range(layers)]
+    return {"architecture": "Ribovik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "layers": entries}
+
+
+def spread_routing(eng: Engine, seed: int = 0) -> None:
+    """Random weights as the engine draws them (all small, corrections all near 1) send every
+    token to the same experts.  A router with large weights and no correction spreads the
+    tokens over the experts, as a trained one does."""
+    g = torch.Generator(device=eng.device).manual_seed(seed)
+    for block in eng.model.blocks:
+        ff = getattr(block, "feed_forward", None)
+        if ff is not None and getattr(ff, "w_router", None) is not None:
+            ff.w_router.copy_(torch.randn(ff.w_router.shape, generator=g, device=eng.device).to(ff.w_router.dtype))
+            if ff.correction is not None:
+                ff.correction.zero_()
+            if ff._tiled.get("router") is not None:
+                from .parts.linear import tiled_copy
+                from . import kernels as K
+                ff._tiled["router"] = tiled_copy(ff.runtime, ff.w_router, K.LINEAR_PARTS)
+                ff.runtime.tensors_changed()
+
+
 def measure_design_pair(sizes: dict, dtype: str, batches=(1, 8), context: int = 2048, prompt: int = 2048,
-                        steps: int = 64, delta_every: int = 4) -> dict:
-    """Prefill and decode throughput of a Nusilix model and of a Llama model of the same layer
-    sizes, one after the other on this GPU."""
+                        steps: int = 64, delta_every: int = 4, design: str = "nusilix", design_sizes=None) -> dict:
+    """Prefill and decode throughput of a model of ``design`` ("nusilix", "ribovik") and of a
+    Llama model of the same layer sizes, one after the other on this GPU."""
     import gc
     out = {}
-    for name, cfg in (("nusilix", nusilix_config(delta_every=delta_every, **sizes)), ("llama", llama_config(**sizes))):
+    if design == "ribovik":
+        first = ribovik_config(**sizes, **(design_sizes or {}), chunk=max(4096, context + 64))
+    else:
+        first = nusilix_config(delta_every=delta_every, **sizes)
+    for name, cfg in ((design, first), ("llama", llama_config(**sizes))):
         eng = make_engine(cfg, dtype, max_tokens=max(batches) * context + 2 * prompt, max_model_len=context + 64,
                           max_requests=max(batches))
+        spread_routing(eng)
         res = {"weights_GB": round(eng.model.weight_bytes() / 1e9, 3)}
         pms = measure_prefill(eng, prompt)
         flops = eng.model.step_flops(prompt, prompt * (prompt + 1) / 2.0, 1)

@@ -47,6 +47,7 @@ static const Op kOps[] = {
     KLLM_CMD_OP(kllm_moe_route),
     KLLM_CMD_OP(kllm_moe_plan),
     KLLM_CMD_OP(kllm_moe_expert),
+    KLLM_CMD_OP(kllm_moe_expert_rows),
     KLLM_CMD_OP(kllm_moe_combine),
 };
 constexpr int kNumOps = (int)(sizeof(kOps) / sizeof(kOps[0]));

@@ -377,6 +377,11 @@ int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int* sorted
 int kllm_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
                     int max_tiles, int top, int m, int k, int mode, int act, float limit, float alpha,
                     int dtype, hipStream_t stream);
+/* kllm_moe_expert without tiles, entry by entry (idx [entries] names each entry's expert; those
+ * from E on are skipped): for decode batches. */
+int kllm_moe_expert_rows(const void* x, const void* w, void* out, const int* idx, int entries, int E,
+                         int top, int m, int k, int mode, int act, float limit, float alpha, int dtype,
+                         hipStream_t stream);
 int kllm_moe_combine(const float* y, const void* xin, const int* idx, const float* wgt, const float* shared,
                      int ns, long shared_stride, float* out, int n, int d, int top, int E, int dtype,
                      hipStream_t stream);

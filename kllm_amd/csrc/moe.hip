@@ -4,10 +4,12 @@
 //   kllm_moe_route    per token: softmax of the router's sums over all experts, the `top` largest
 //                     of (score + correction), their scores divided by their sum
 //   kllm_moe_plan     the (token, choice) entries grouped by expert, and a list of tiles of up to
-//                     32 entries of one expert (a fixed number of tiles, the unused ones empty)
-//   kllm_moe_expert   one tile's product with its expert's weights on the matrix cores (32 x 32
-//                     per wave, 32-bit or bfloat16 operands straight from memory): gate and up
-//                     with the gate in the epilogue, or down
+//                     64 entries of one expert (a fixed number of tiles, the unused ones empty)
+//   kllm_moe_expert   one tile's product with its expert's weights on the matrix cores (64 rows by
+//                     64 columns a workgroup through LDS, 32-bit or bfloat16 operands): gate and
+//                     up with the gate in the epilogue, or down
+//   kllm_moe_expert_rows  the same products entry by entry, for decode batches: no plan, a wave
+//                     per two columns, the whole of K of a row in flight at once
 //   kllm_moe_combine  per token the weighted sum of its choices' outputs, in the order of the
 //                     choices; an expert beyond the last real one is the identity (its output is
 //                     the feed-forward's input); plus the sums of a shared expert
@@ -21,12 +23,17 @@
 
 namespace kllm {
 
-constexpr int kMoeTileRows = 32;
+constexpr int kMoeTileRows = 64;
+constexpr int kMaxTop = 128;        // experts a token may use at most
+constexpr int kMaxRouted = 4096;    // experts a router may choose from at most
 
-__global__ void moe_route_kernel(const float* __restrict__ z, int nsplit, long split_stride,
-                                 const float* __restrict__ correction, int n, int R, int top, int* __restrict__ idx,
-                                 float* __restrict__ wgt) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+// One wave per token; a lane takes the experts lane, lane + 64, ...  The largest of a set is
+// found lane by lane and then across the wave, the lower expert winning a tie.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, int nsplit, long split_stride,
+                                                        const float* __restrict__ correction, int n, int R, int top,
+                                                        int* __restrict__ idx, float* __restrict__ wgt) {
+  const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
   if (t >= n) return;
   auto z_at = [&](int e) {
     float v = 0.f;
@@ -34,17 +41,19 @@ __global__ void moe_route_kernel(const float* __restrict__ z, int nsplit, long s
     return v;
   };
   float m = -INFINITY;
-  for (int e = 0; e < R; ++e) m = fmaxf(m, z_at(e));
+  for (int e = lane; e < R; e += kWave) m = fmaxf(m, z_at(e));
+  m = wave_max(m);
   float den = 0.f;
-  for (int e = 0; e < R; ++e) den += expf(z_at(e) - m);
+  for (int e = lane; e < R; e += kWave) den += expf(z_at(e) - m);
+  den = wave_sum(den);
   float picked = 0.f;
+  float mine[kMaxTop / kWave] = {};
+  unsigned long long taken = 0;      // bit i: this lane's expert lane + 64 i is chosen already
   for (int k = 0; k < top; ++k) {
-    int best = 0;
+    int best = R;
     float best_choice = -INFINITY, best_score = 0.f;
-    for (int e = 0; e < R; ++e) {
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken |= idx[(long)t * top + j] == e;
-      if (taken) continue;
+    for (int e = lane; e < R; e += kWave) {
+      if ((taken >> (e / kWave)) & 1) continue;
       const float s = expf(z_at(e) - m) / den;
       const float c = correction ? s + correction[e] : s;
       if (c > best_choice) {
@@ -53,12 +62,23 @@ __global__ void moe_route_kernel(const float* __restrict__ z, int nsplit, long s
         best = e;
       }
     }
-    idx[(long)t * top + k] = best;
-    wgt[(long)t * top + k] = best_score;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      const float oc = __shfl_xor(best_choice, off, kWave), os = __shfl_xor(best_score, off, kWave);
+      const int ob = __shfl_xor(best, off, kWave);
+      if (oc > best_choice || (oc == best_choice && ob < best)) {
+        best_choice = oc;
+        best_score = os;
+        best = ob;
+      }
+    }
+    if (best % kWave == lane) taken |= 1ull << (best / kWave);
+    if (lane == 0) idx[(long)t * top + k] = best;
+    if (lane == k % kWave) mine[k / kWave] = best_score;      // lane k keeps the k-th score until the sum is known
     picked += best_score;
   }
   const float inv = 1.f / (picked + 1e-20f);
-  for (int k = 0; k < top; ++k) wgt[(long)t * top + k] *= inv;
+  for (int k = lane; k < top; k += kWave) wgt[(long)t * top + k] = mine[k / kWave] * inv;
 }
 
 // One workgroup.  tiles: [max_tiles][3] = (expert, first place in `sorted`, entries).
@@ -131,9 +151,15 @@ __device__ __forceinline__ typename MoeOperand<T>::type moe_chunk(const T* __res
 // MODE 0: X is the feed-forward's input [tokens, K]; W [E][2 M][K], an expert's gate rows, then its
 //         up rows; out [entries, M] in T: the gated activation.
 // MODE 1: X is [entries, K]; W [E][M][K]; out [entries, M] float32.
-// Grid (tiles, column blocks of 128); a wave takes 32 columns.  A lane's share of K: of every
-// 128 bytes of a row, lanes 0-31 take the first 64 for their row and lanes 32-63 the other 64,
-// four products of 16 bytes each; both operands are cut alike, which is all a product asks.
+// Grid (tiles, column blocks of 64).  A workgroup's four waves share a tile of 64 rows of X by 64
+// columns (MODE 0: 64 gate rows and 64 up rows of W), 32 x 32 each.  128 bytes of K of every row
+// pass through LDS in two buffers: a thread asks memory for its 16-byte pieces of the next step,
+// multiplies this step out of LDS, then puts the pieces down behind it.  Rows lie 144 bytes
+// apart, so that the 16 lanes of a read meet 16 different groups of banks.  Which 16 bytes of
+// K a lane multiplies in which of a step's four products is the same for both operands, which
+// is all a product asks.
+constexpr int kMoeRowBytes = 144;
+
 template <typename T, int MODE>
 __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ out_, const int* __restrict__ sorted,
@@ -141,62 +167,145 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X
                                                          float limit, float alpha) {
   typedef typename MoeOperand<T>::type op_t;
   constexpr int EPC = 16 / sizeof(T);
+  constexpr int NB = MODE == 0 ? 2 : 1;           // blocks of 64 rows of W: gate (and up)
+  constexpr int AROWS = kMoeTileRows, BROWS = 64 * NB;
+  constexpr int STAGE = (AROWS + BROWS) * kMoeRowBytes;
+  constexpr int STEP = 8 * EPC;                   // elements of 128 bytes
+  extern __shared__ __attribute__((aligned(16))) unsigned char moe_lds[];   // [2][STAGE]
   const int tile = blockIdx.x;
   const int count = tiles[3 * tile + 2];
   if (count == 0) return;
   const int expert = tiles[3 * tile], start = tiles[3 * tile + 1];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int c0 = (blockIdx.y * 4 + wave) * 32;
+  const int c0 = blockIdx.y * 64;
   if (c0 >= M) return;
-  const int r = lane % 32, half = lane / 32;
-  const int entry = sorted[start + (r < count ? r : 0)];
-  const T* xrow = X + (long)(MODE == 0 ? entry / top : entry) * K;
-  const int wr = min(c0 + r, M - 1);
-  const T* wbase = W + (long)expert * (MODE == 0 ? 2 : 1) * M * K;
-  const T* w0 = wbase + (long)wr * K;
-  const T* w1 = wbase + (long)(M + wr) * K;      // MODE 0: the up row
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wr = wave / 2, wc = wave % 2, r = lane % 32, half = lane / 32;
   const bool vec = K % EPC == 0;
+  const T* wbase = W + (long)expert * NB * M * K;
+  // what this thread brings in: piece `ch` of rows tid / 8 + 32 i of X and of W
+  const int ch = tid % 8, row0 = tid / 8;
+  const T* arow[AROWS / 32];
+  const T* brow[BROWS / 32];
+#pragma unroll
+  for (int i = 0; i < AROWS / 32; ++i) {
+    const int entry = sorted[start + min(row0 + 32 * i, count - 1)];
+    arow[i] = X + (long)(MODE == 0 ? entry / top : entry) * K;
+  }
+#pragma unroll
+  for (int i = 0; i < BROWS / 32; ++i) {
+    const int row = row0 + 32 * i;                // 0 .. 63: gate (or the one product), 64 .. 127: up
+    brow[i] = wbase + ((long)(row / 64) * M + min(c0 + row % 64, M - 1)) * K;
+  }
+  op_t ra[AROWS / 32], rb[BROWS / 32];
+  auto load = [&](int k) {
+    const int k0 = k + ch * EPC;
+#pragma unroll
+    for (int i = 0; i < AROWS / 32; ++i) ra[i] = moe_chunk<T>(arow[i], k0, K, vec);
+#pragma unroll
+    for (int i = 0; i < BROWS / 32; ++i) rb[i] = moe_chunk<T>(brow[i], k0, K, vec);
+  };
+  auto put = [&](int buf) {
+    unsigned char* base = moe_lds + buf * STAGE + ch * 16;
+#pragma unroll
+    for (int i = 0; i < AROWS / 32; ++i) *reinterpret_cast<op_t*>(base + (row0 + 32 * i) * kMoeRowBytes) = ra[i];
+#pragma unroll
+    for (int i = 0; i < BROWS / 32; ++i)
+      *reinterpret_cast<op_t*>(base + (AROWS + row0 + 32 * i) * kMoeRowBytes) = rb[i];
+  };
   floatx16 acc0, acc1;
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.f;
-  constexpr int STEP = 8 * EPC;                  // elements of 128 bytes
-  op_t a[4], b0[4], b1[4];
-  auto load = [&](int k) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int k0 = k + (half * 4 + i) * EPC;
-      a[i] = moe_chunk<T>(xrow, k0, K, vec);
-      b0[i] = moe_chunk<T>(w0, k0, K, vec);
-      if (MODE == 0) b1[i] = moe_chunk<T>(w1, k0, K, vec);
-    }
-  };
   load(0);
-  for (int k = 0; k < K; k += STEP) {
-    op_t ca[4], cb0[4], cb1[4];
+  put(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k = 0; k < K; k += STEP, buf ^= 1) {
+    const bool more = k + STEP < K;
+    if (more) load(k + STEP);
+    const unsigned char* base = moe_lds + buf * STAGE;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      ca[i] = a[i];
-      cb0[i] = b0[i];
-      if (MODE == 0) cb1[i] = b1[i];
+      const int piece = (2 * i + half) * 16;
+      const op_t a = *reinterpret_cast<const op_t*>(base + (wr * 32 + r) * kMoeRowBytes + piece);
+      const op_t b0 = *reinterpret_cast<const op_t*>(base + (AROWS + wc * 32 + r) * kMoeRowBytes + piece);
+      acc0 = moe_mfma(a, b0, acc0);
+      if (MODE == 0) {
+        const op_t b1 = *reinterpret_cast<const op_t*>(base + (AROWS + 64 + wc * 32 + r) * kMoeRowBytes + piece);
+        acc1 = moe_mfma(a, b1, acc1);
+      }
     }
-    if (k + STEP < K) load(k + STEP);            // the next 128 bytes are on their way during the products
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      acc0 = moe_mfma(ca[i], cb0[i], acc0);
-      if (MODE == 0) acc1 = moe_mfma(ca[i], cb1[i], acc1);
-    }
+    if (more) put(buf ^ 1);
+    __syncthreads();
   }
-  const int c = c0 + r;
+  const int c = c0 + wc * 32 + r;
   if (c >= M) return;
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
-    const int row = 8 * (e / 4) + 4 * half + e % 4;
+    const int row = wr * 32 + 8 * (e / 4) + 4 * half + e % 4;
     if (row >= count) continue;
     const long dst = (long)sorted[start + row] * M + c;
     if (MODE == 0)
       reinterpret_cast<T*>(out_)[dst] = from_f32<T>(gated(acc0[e], acc1[e], act, limit, alpha));
     else
       reinterpret_cast<float*>(out_)[dst] = acc0[e];
+  }
+}
+
+// The same products for few entries (decode batches), without tiles or a plan: a workgroup takes
+// one entry and eight columns of its expert, two to a wave; a lane's share of K is every 64th
+// piece of 16 bytes, all of a row's pieces asked for at once.  idx [entries]: the entry's expert
+// (entries of experts from E on are skipped).
+template <typename T>
+__device__ __forceinline__ float moe_dot(typename MoeOperand<T>::type a, typename MoeOperand<T>::type b, float acc) {
+  constexpr int EPC = 16 / sizeof(T);
+#pragma unroll
+  for (int j = 0; j < EPC; ++j) acc = fmaf(to_f32((T)a[j]), to_f32((T)b[j]), acc);
+  return acc;
+}
+
+constexpr int kGemvCols = 2;       // columns a wave
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void moe_gemv_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                       void* __restrict__ out_, const int* __restrict__ idx, int E,
+                                                       int top, int M, int K, int act, float limit, float alpha) {
+  constexpr int EPC = 16 / sizeof(T);
+  const int entry = blockIdx.x;
+  const int expert = idx[entry];
+  if (expert >= E) return;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int c0 = (blockIdx.y * 4 + wave) * kGemvCols;
+  if (c0 >= M) return;
+  const T* xrow = X + (long)(MODE == 0 ? entry / top : entry) * K;
+  const T* wbase = W + (long)expert * (MODE == 0 ? 2 : 1) * M * K;
+  const bool vec = K % EPC == 0;
+  float g[kGemvCols], u[kGemvCols];
+#pragma unroll
+  for (int c = 0; c < kGemvCols; ++c) g[c] = u[c] = 0.f;
+#pragma unroll 2
+  for (int k = lane * EPC; k < K; k += kWave * EPC) {
+    const auto a = moe_chunk<T>(xrow, k, K, vec);
+#pragma unroll
+    for (int c = 0; c < kGemvCols; ++c) {
+      const int col = min(c0 + c, M - 1);
+      g[c] = moe_dot<T>(a, moe_chunk<T>(wbase + (long)col * K, k, K, vec), g[c]);
+      if (MODE == 0) u[c] = moe_dot<T>(a, moe_chunk<T>(wbase + (long)(M + col) * K, k, K, vec), u[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kGemvCols; ++c) {
+    g[c] = wave_sum(g[c]);
+    if (MODE == 0) u[c] = wave_sum(u[c]);
+  }
+  if (lane != 0) return;
+#pragma unroll
+  for (int c = 0; c < kGemvCols; ++c) {
+    if (c0 + c >= M) continue;
+    const long dst = (long)entry * M + c0 + c;
+    if (MODE == 0)
+      reinterpret_cast<T*>(out_)[dst] = from_f32<T>(gated(g[c], u[c], act, limit, alpha));
+    else
+      reinterpret_cast<float*>(out_)[dst] = g[c];
   }
 }
 
@@ -227,9 +336,9 @@ extern "C" int kllm_moe_tile_rows(void) { return kMoeTileRows; }
 extern "C" int kllm_moe_route(const float* z, int nsplit, long split_stride, const float* correction, int n, int R,
                               int top, int* idx, float* wgt, hipStream_t stream) {
   KLLM_REQUIRE(z && idx && wgt, "moe_route: null pointer");
-  KLLM_REQUIRE(n > 0 && R > 0 && top > 0 && top <= R && nsplit >= 1, "moe_route: bad sizes n=%d experts=%d top=%d", n, R,
-               top);
-  hipLaunchKernelGGL(moe_route_kernel, dim3(ceil_div(n, 64)), dim3(64), 0, stream, z, nsplit, split_stride, correction,
+  KLLM_REQUIRE(n > 0 && R > 0 && R <= kMaxRouted && top > 0 && top <= R && top <= kMaxTop && nsplit >= 1,
+               "moe_route: bad sizes n=%d experts=%d (up to %d) top=%d (up to %d)", n, R, kMaxRouted, top, kMaxTop);
+  hipLaunchKernelGGL(moe_route_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, stream, z, nsplit, split_stride, correction,
                      n, R, top, idx, wgt);
   KLLM_CHECK_LAUNCH("moe_route");
   return 0;
@@ -256,9 +365,10 @@ extern "C" int kllm_moe_expert(const void* x, const void* w, void* out, const in
   KLLM_REQUIRE(mode == 0 || mode == 1, "moe_expert: mode %d", mode);
   KLLM_REQUIRE(mode == 1 || gated_known(act), "moe_expert: unknown activation %d", act);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "moe_expert: unknown dtype %d", dtype);
-  const dim3 grid(max_tiles, ceil_div(m, 128));
-#define KLLM_MOE(T, MODE)                                                                                          \
-  hipLaunchKernelGGL((moe_expert_kernel<T, MODE>), grid, dim3(256), 0, stream, (const T*)x, (const T*)w, out, sorted, \
+  const dim3 grid(max_tiles, ceil_div(m, 64));
+  const size_t lds = (size_t)2 * (kMoeTileRows + (mode == 0 ? 128 : 64)) * kMoeRowBytes;
+#define KLLM_MOE(T, MODE)                                                                                            \
+  hipLaunchKernelGGL((moe_expert_kernel<T, MODE>), grid, dim3(256), lds, stream, (const T*)x, (const T*)w, out, sorted, \
                      tiles, top, m, k, act, limit, alpha)
   if (dtype == DT_F32) {
     if (mode == 0) KLLM_MOE(float, 0); else KLLM_MOE(float, 1);
@@ -267,6 +377,29 @@ extern "C" int kllm_moe_expert(const void* x, const void* w, void* out, const in
   }
 #undef KLLM_MOE
   KLLM_CHECK_LAUNCH("moe_expert");
+  return 0;
+}
+
+extern "C" int kllm_moe_expert_rows(const void* x, const void* w, void* out, const int* idx, int entries, int E,
+                                    int top, int m, int k, int mode, int act, float limit, float alpha, int dtype,
+                                    hipStream_t stream) {
+  KLLM_REQUIRE(x && w && out && idx, "moe_expert_rows: null pointer");
+  KLLM_REQUIRE(entries > 0 && entries <= 65535 && E > 0 && top > 0 && m > 0 && k > 0,
+               "moe_expert_rows: bad sizes entries=%d E=%d top=%d m=%d k=%d", entries, E, top, m, k);
+  KLLM_REQUIRE(mode == 0 || mode == 1, "moe_expert_rows: mode %d", mode);
+  KLLM_REQUIRE(mode == 1 || gated_known(act), "moe_expert_rows: unknown activation %d", act);
+  KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "moe_expert_rows: unknown dtype %d", dtype);
+  const dim3 grid(entries, ceil_div(m, 4 * kGemvCols));
+#define KLLM_MOE(T, MODE)                                                                                      \
+  hipLaunchKernelGGL((moe_gemv_kernel<T, MODE>), grid, dim3(256), 0, stream, (const T*)x, (const T*)w, out, idx, E, \
+                     top, m, k, act, limit, alpha)
+  if (dtype == DT_F32) {
+    if (mode == 0) KLLM_MOE(float, 0); else KLLM_MOE(float, 1);
+  } else {
+    if (mode == 0) KLLM_MOE(bf16_t, 0); else KLLM_MOE(bf16_t, 1);
+  }
+#undef KLLM_MOE
+  KLLM_CHECK_LAUNCH("moe_expert_rows");
   return 0;
 }
 

@@ -121,6 +121,7 @@ def _declare(lib):
         "kllm_moe_route": [P, I, L, P, I, I, I, P, P, P],
         "kllm_moe_plan": [P, I, I, I, P, P, P],
         "kllm_moe_expert": [P, P, P, P, P, I, I, I, I, I, I, F, F, I, P],
+        "kllm_moe_expert_rows": [P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "kllm_moe_combine": [P, P, P, P, P, I, L, P, I, I, I, I, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
         "kllm_attn_decode_slices": [I, I, I, I, I, I],
@@ -166,7 +167,7 @@ LAUNCHING = ("kllm_embed", "kllm_add_rmsnorm", "kllm_rope_tables", "kllm_rope_ap
              "kllm_attn_decode", "kllm_attn_prefill", "kllm_sample", "kllm_gemm_act", "kllm_add_sinusoid", "kllm_unary_act",
              "kllm_group_norm_add", "kllm_qk_norm_append", "kllm_delta_prep", "kllm_delta_scan", "kllm_delta_out",
              "kllm_norm_residual", "kllm_rope_tables_freq", "kllm_qkv_norm_append", "kllm_gate_bias", "kllm_moe_route",
-             "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_combine")
+             "kllm_moe_plan", "kllm_moe_expert", "kllm_moe_expert_rows", "kllm_moe_combine")
 DYNAMIC_ARGS = {"kllm_attn_prefill": (18, 19)}     # arguments that may be a StepValue
 STRUCT_ARGS = {"kllm_gemv_plain": (7,), "kllm_gemv_swiglu": (8,), "kllm_gemv_rope_append": (17,),
                "kllm_fused_linear": (2,)}
@@ -1463,6 +1464,23 @@ def moe_expert(x, w, out, sorted_entries, tiles, top, mode, act=ACT_SILU, limit=
             _ptr(sorted_entries, "moe_expert sorted", torch.int32), _ptr(tiles, "moe_expert tiles", torch.int32),
             tiles.shape[0], int(top), m, k, int(mode), int(act), float(limit), float(alpha), dtype_code(x.dtype),
             _stream())
+
+
+MOE_ROWS_BEST_ENTRIES = 16     # (token, choice) pairs up to which the entry-by-entry products beat the tiles
+
+
+def moe_expert_rows(x, w, out, idx, experts, mode, act=ACT_SILU, limit=0.0, alpha=1.0):
+    """``moe_expert`` entry by entry, without a plan: idx int32 [tokens, top] names each entry's
+    expert; entries of experts from ``experts`` on are skipped."""
+    k, m, top = x.shape[1], out.shape[1], idx.shape[1]
+    entries = idx.numel()
+    if (w.dim() != 3 or w.shape[2] != k or w.shape[1] != (2 * m if mode == 0 else m) or w.dtype != x.dtype
+            or out.dtype != (x.dtype if mode == 0 else torch.float32) or out.shape[0] != entries
+            or x.shape[0] != (entries // top if mode == 0 else entries)):
+        raise KernelError(f"moe_expert_rows: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    _launch("kllm_moe_expert_rows", "moe_expert_rows", _ptr(x, "moe_expert_rows x"), _ptr(w, "moe_expert_rows w"),
+            _ptr(out, "moe_expert_rows out"), _ptr(idx, "moe_expert_rows idx", torch.int32), entries, int(experts), top,
+            m, k, int(mode), int(act), float(limit), float(alpha), dtype_code(x.dtype), _stream())
 
 
 def moe_combine(y, xin, idx, wgt, out, experts, shared=None):

@@ -118,13 +118,18 @@ class RoutedExperts(Part):
         idx = ctx.buf("moe.idx", (n, top), torch.int32)
         wgt = ctx.buf("moe.wgt", (n, top), torch.float32)
         K.moe_route(z, self.correction, idx, wgt)
-        tiles = ctx.buf("moe.tiles", (K.moe_max_tiles(n * top, self.experts), 3), torch.int32)
-        order = ctx.buf("moe.sorted", (n * top,), torch.int32)
-        K.moe_plan(idx, self.experts, order, tiles)
         h = ctx.buf("moe.h", (n * top, f), dtype)
-        K.moe_expert(xn, self.w_gu, h, order, tiles, top, 0, self.act, self.limit, self.alpha)
         y = ctx.buf("moe.y", (n * top, d), torch.float32)
-        K.moe_expert(h, self.w_down, y, order, tiles, top, 1)
+        if n * top <= K.MOE_ROWS_BEST_ENTRIES and not self.runtime.options.get("moe_tiles_only"):
+            # a decode batch: entry by entry, every chosen expert's rows streamed once
+            K.moe_expert_rows(xn, self.w_gu, h, idx, self.experts, 0, self.act, self.limit, self.alpha)
+            K.moe_expert_rows(h, self.w_down, y, idx, self.experts, 1)
+        else:
+            tiles = ctx.buf("moe.tiles", (K.moe_max_tiles(n * top, self.experts), 3), torch.int32)
+            order = ctx.buf("moe.sorted", (n * top,), torch.int32)
+            K.moe_plan(idx, self.experts, order, tiles)
+            K.moe_expert(xn, self.w_gu, h, order, tiles, top, 0, self.act, self.limit, self.alpha)
+            K.moe_expert(h, self.w_down, y, order, tiles, top, 1)
         shared = None
         if self.shared_intermediate:
             hs = gated_hidden(ctx, xn, self.w_shared_gu, self.shared_intermediate, "moe.shared",
