@@ -20,15 +20,51 @@ namespace kllm {
 
 constexpr int kRowThreads = 256;
 
-// One workgroup per row, the row's sums kept in LDS between the two passes.
-template <typename TOUT>
+// One workgroup per row.  PER > 0: a thread keeps its PER elements of the row in registers, and
+// everything it reads (the sums' slices, the bias, the stream, the weight) is asked for before
+// the first use, so that a row costs one trip to memory (decode batches: one row, one workgroup).
+// PER == 0: rows of any length, the row's sums kept in LDS between the two passes.
+template <typename TOUT, int PER>
 __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int nsplit, long split_stride,
     const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps) {
-  extern __shared__ float row_lds[];      // [d]
+  extern __shared__ float row_lds[];      // [d] (PER == 0)
   __shared__ float red[16];
   const long r = blockIdx.x;
   float* xr = x + r * d;
+  if constexpr (PER > 0) {
+    float v[PER], xv[PER], wv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + kRowThreads * j;
+      const bool ok = i < d;
+      const int ii = ok ? i : 0;
+      xv[j] = xr[ii];
+      wv[j] = w[ii];
+      float t = 0.f;
+      if (delta) {
+        for (int s = 0; s < nsplit; ++s) t += delta[s * split_stride + r * d + ii];
+        if (bias) t += bias[ii];
+      } else {
+        t = xv[j];
+      }
+      v[j] = ok ? t : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) ss = fmaf(v[j], v[j], ss);
+    const float rstd = 1.f / sqrtf(block_sum(ss, red) / (float)d + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int i = threadIdx.x + kRowThreads * j;
+      if (i >= d) continue;
+      const float y = v[j] * rstd * wv[j];
+      const float nv = delta ? xv[j] + y : y;
+      xr[i] = nv;
+      if (out) out[r * d + i] = from_f32<TOUT>(nv);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += kRowThreads) {
     float v;
@@ -162,13 +198,21 @@ extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long
   KLLM_REQUIRE(!delta || nsplit >= 1, "norm_residual: nsplit %d", nsplit);
   KLLM_REQUIRE(delta || !bias, "norm_residual: a bias goes with sums");
   KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "norm_residual: unknown dtype %d", out_dtype);
-  const size_t lds = (size_t)d * sizeof(float);
-  if (out && out_dtype == DT_BF16)
-    hipLaunchKernelGGL(norm_residual_kernel<bf16_t>, dim3(n), dim3(kRowThreads), lds, stream, x, delta, nsplit,
-                       split_stride, bias, weight, (bf16_t*)out, d, eps);
-  else
-    hipLaunchKernelGGL(norm_residual_kernel<float>, dim3(n), dim3(kRowThreads), lds, stream, x, delta, nsplit,
-                       split_stride, bias, weight, (float*)out, d, eps);
+#define KLLM_NR(TOUT, PER)                                                                                    \
+  hipLaunchKernelGGL((norm_residual_kernel<TOUT, PER>), dim3(n), dim3(kRowThreads),                           \
+                     PER ? 0 : (size_t)d * sizeof(float), stream, x, delta, nsplit, split_stride, bias, weight, \
+                     (TOUT*)out, d, eps)
+  const bool bf = out && out_dtype == DT_BF16;
+  if (d <= 4 * kRowThreads) {
+    if (bf) KLLM_NR(bf16_t, 4); else KLLM_NR(float, 4);
+  } else if (d <= 8 * kRowThreads) {
+    if (bf) KLLM_NR(bf16_t, 8); else KLLM_NR(float, 8);
+  } else if (d <= 16 * kRowThreads) {
+    if (bf) KLLM_NR(bf16_t, 16); else KLLM_NR(float, 16);
+  } else {
+    if (bf) KLLM_NR(bf16_t, 0); else KLLM_NR(float, 0);
+  }
+#undef KLLM_NR
   KLLM_CHECK_LAUNCH("norm_residual");
   return 0;
 }
