@@ -165,7 +165,7 @@ def test_recorded_commands_are_copied_and_added_with_their_step_values():
         n_args = K._ops()["kllm_attn_prefill"].nargs
         dynamic = K._ops()["kllm_attn_prefill"].dynamic
         args = [1000 + i for i in range(n_args)]
-        args[14] = 0.125                                              # the scale, a float
+        args[dynamic[0] - 2] = 0.125                                  # the scale, a float, two in front of the step's values
         args[dynamic[0]], args[dynamic[1]] = K.StepValue(777, "keys.total"), K.StepValue(55, "keys.longest")
         K._launch("kllm_attn_prefill", "before", *args)
         first = rec.at
