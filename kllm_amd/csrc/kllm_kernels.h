@@ -337,10 +337,15 @@ int kllm_delta_out(const float* o, const float* gate, const float* weight, float
 /* Layers whose norm stands behind the sub-layer.  x [n, d] float32.  With sums (`delta`, float32
  * [nsplit][n][d], plus `bias` [d] or null): x += weight * N(delta + bias); without: x = weight *
  * N(x); N(v) = v / sqrt(mean(v^2) + eps).  `out` (or null) receives the new rows of x in
- * `out_dtype`, for the next product. */
+ * `out_dtype`, for the next product.
+ * The sums may also be those of a routed feed-forward's chosen experts, not yet added up
+ * (`chosen_y` [n * top][d], null: none): then the row is the sum over the token's choices of
+ * chosen_wgt * (chosen_idx < E ? chosen_y : chosen_x, the feed-forward's input [n][d]) + delta's
+ * slices (a shared expert's; may be null) + bias. */
 int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
                        const float* weight, void* out, int out_dtype, int n, int d, float eps,
-                       hipStream_t stream);
+                       const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
+                       const float* chosen_wgt, int top, int E, hipStream_t stream);
 /* cos/sin [n][half] = factor * cos/sin(positions[t] * freq[i]), the angle in double. */
 int kllm_rope_tables_freq(float* cos_t, float* sin_t, const int* positions, const double* freq, int n,
                           int half, double factor, hipStream_t stream);
@@ -364,7 +369,8 @@ int kllm_gate_bias(const float* gu, int nsplit, long split_stride, const float* 
  * idx/wgt [n][top] receive the `top` experts with the largest softmax(z) + correction (null: none)
  * and their softmax scores divided by their sum.  plan: the entries (token * top + choice) whose
  * expert is below E, grouped by expert into `sorted`, and `tiles` [max_tiles][3] = (expert, first
- * place in sorted, entries <= kllm_moe_tile_rows()); max_tiles >= ceil(entries / rows) + E.
+ * place in sorted, entries <= tile_rows); tile_rows is kllm_moe_tile_rows() or twice that (the
+ * same in plan and expert); max_tiles >= ceil(entries / tile_rows) + E.
  * expert, mode 0: out [entries][m] (dtype) = gated(gate, up) of x [tokens][k] against w [E][2 m][k];
  * mode 1: out [entries][m] float32 = x [entries][k] against w [E][m][k].  combine: out [n][d] =
  * sum over a token's choices of wgt * (expert < E ? y [entries][d] : xin [n][d]) + the slices of
@@ -372,11 +378,11 @@ int kllm_gate_bias(const float* gu, int nsplit, long split_stride, const float* 
 int kllm_moe_tile_rows(void);
 int kllm_moe_route(const float* z, int nsplit, long split_stride, const float* correction, int n, int R,
                    int top, int* idx, float* wgt, hipStream_t stream);
-int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int* sorted, int* tiles,
+int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int tile_rows, int* sorted, int* tiles,
                   hipStream_t stream);
 int kllm_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
-                    int max_tiles, int top, int m, int k, int mode, int act, float limit, float alpha,
-                    int dtype, hipStream_t stream);
+                    int max_tiles, int tile_rows, int top, int m, int k, int mode, int act, float limit,
+                    float alpha, int dtype, hipStream_t stream);
 /* kllm_moe_expert without tiles, entry by entry (idx [entries] names each entry's expert; those
  * from E on are skipped): for decode batches. */
 int kllm_moe_expert_rows(const void* x, const void* w, void* out, const int* idx, int entries, int E,

@@ -6,8 +6,8 @@
 //   kllm_moe_plan     the (token, choice) entries grouped by expert, and a list of tiles of up to
 //                     64 entries of one expert (a fixed number of tiles, the unused ones empty)
 //   kllm_moe_expert   one tile's product with its expert's weights on the matrix cores (64 rows by
-//                     64 columns a workgroup through LDS, 32-bit or bfloat16 operands): gate and
-//                     up with the gate in the epilogue, or down
+//                     64 columns a workgroup through LDS, or 128 by 128; 32-bit or bfloat16
+//                     operands): gate and up with the gate in the epilogue, or down
 //   kllm_moe_expert_rows  the same products entry by entry, for decode batches: no plan, a wave
 //                     per two columns, the whole of K of a row in flight at once
 //   kllm_moe_combine  per token the weighted sum of its choices' outputs, in the order of the
@@ -23,7 +23,7 @@
 
 namespace kllm {
 
-constexpr int kMoeTileRows = 64;
+constexpr int kMoeTileRows = 64;     // rows of the small tiles; the large ones have twice as many
 constexpr int kMaxTop = 128;        // experts a token may use at most
 constexpr int kMaxRouted = 4096;    // experts a router may choose from at most
 
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 
 // One workgroup.  tiles: [max_tiles][3] = (expert, first place in `sorted`, entries).
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ idx, int entries, int E, int max_tiles,
-                                                        int* __restrict__ sorted, int* __restrict__ tiles) {
+                                                        int tile_rows, int* __restrict__ sorted, int* __restrict__ tiles) {
   extern __shared__ int plan_lds[];
   int* counts = plan_lds;
   int* offs = plan_lds + E;
@@ -99,10 +99,10 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     int off = 0, nt = 0;
     for (int e = 0; e < E; ++e) {
       offs[e] = off;
-      for (int s = 0; s < counts[e] && nt < max_tiles; s += kMoeTileRows, ++nt) {
+      for (int s = 0; s < counts[e] && nt < max_tiles; s += tile_rows, ++nt) {
         tiles[3 * nt] = e;
         tiles[3 * nt + 1] = off + s;
-        tiles[3 * nt + 2] = min(kMoeTileRows, counts[e] - s);
+        tiles[3 * nt + 2] = min(tile_rows, counts[e] - s);
       }
       off += counts[e];
     }
@@ -151,8 +151,10 @@ __device__ __forceinline__ typename MoeOperand<T>::type moe_chunk(const T* __res
 // MODE 0: X is the feed-forward's input [tokens, K]; W [E][2 M][K], an expert's gate rows, then its
 //         up rows; out [entries, M] in T: the gated activation.
 // MODE 1: X is [entries, K]; W [E][M][K]; out [entries, M] float32.
-// Grid (tiles, column blocks of 64).  A workgroup's four waves share a tile of 64 rows of X by 64
-// columns (MODE 0: 64 gate rows and 64 up rows of W), 32 x 32 each.  128 bytes of K of every row
+// Grid (tiles, column blocks).  A workgroup's four waves share a tile of 64 rows of X by 64
+// columns (MODE 0: 64 gate rows and 64 up rows of W), 32 x 32 each, or of 128 rows by 128 columns
+// (MODE 0: by 64, which is as many rows of W), 64 x 64 each: the larger tile asks the caches for
+// fewer bytes a product, the smaller wastes less where an expert has few rows.  128 bytes of K of every row
 // pass through LDS in two buffers: a thread asks memory for its 16-byte pieces of the next step,
 // multiplies this step out of LDS, then puts the pieces down behind it.  Rows lie 144 bytes
 // apart, so that the 16 lanes of a read meet 16 different groups of banks.  Which 16 bytes of
@@ -160,15 +162,15 @@ __device__ __forceinline__ typename MoeOperand<T>::type moe_chunk(const T* __res
 // is all a product asks.
 constexpr int kMoeRowBytes = 144;
 
-template <typename T, int MODE>
+template <typename T, int MODE, int MI, int NJ>    // a workgroup's tile: 64 MI rows by 64 NJ columns
 __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ out_, const int* __restrict__ sorted,
                                                          const int* __restrict__ tiles, int top, int M, int K, int act,
                                                          float limit, float alpha) {
   typedef typename MoeOperand<T>::type op_t;
   constexpr int EPC = 16 / sizeof(T);
-  constexpr int NB = MODE == 0 ? 2 : 1;           // blocks of 64 rows of W: gate (and up)
-  constexpr int AROWS = kMoeTileRows, BROWS = 64 * NB;
+  constexpr int NB = MODE == 0 ? 2 : 1;           // blocks of rows of W: gate (and up)
+  constexpr int AROWS = 64 * MI, BCOLS = 64 * NJ, BROWS = BCOLS * NB;
   constexpr int STAGE = (AROWS + BROWS) * kMoeRowBytes;
   constexpr int STEP = 8 * EPC;                   // elements of 128 bytes
   extern __shared__ __attribute__((aligned(16))) unsigned char moe_lds[];   // [2][STAGE]
@@ -176,10 +178,10 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X
   const int count = tiles[3 * tile + 2];
   if (count == 0) return;
   const int expert = tiles[3 * tile], start = tiles[3 * tile + 1];
-  const int c0 = blockIdx.y * 64;
+  const int c0 = blockIdx.y * BCOLS;
   if (c0 >= M) return;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wr = wave / 2, wc = wave % 2, r = lane % 32, half = lane / 32;
+  const int wr = wave / 2, wc = wave % 2, r = lane % 32, half = lane / 32;   // a wave: 32 MI rows by 32 NJ columns
   const bool vec = K % EPC == 0;
   const T* wbase = W + (long)expert * NB * M * K;
   // what this thread brings in: piece `ch` of rows tid / 8 + 32 i of X and of W
@@ -193,8 +195,8 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X
   }
 #pragma unroll
   for (int i = 0; i < BROWS / 32; ++i) {
-    const int row = row0 + 32 * i;                // 0 .. 63: gate (or the one product), 64 .. 127: up
-    brow[i] = wbase + ((long)(row / 64) * M + min(c0 + row % 64, M - 1)) * K;
+    const int row = row0 + 32 * i;                // the first BCOLS: gate (or the one product), then up
+    brow[i] = wbase + ((long)(row / BCOLS) * M + min(c0 + row % BCOLS, M - 1)) * K;
   }
   op_t ra[AROWS / 32], rb[BROWS / 32];
   auto load = [&](int k) {
@@ -212,9 +214,15 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X
     for (int i = 0; i < BROWS / 32; ++i)
       *reinterpret_cast<op_t*>(base + (AROWS + row0 + 32 * i) * kMoeRowBytes) = rb[i];
   };
-  floatx16 acc0, acc1;
+  floatx16 acc[MI][NJ][NB];
 #pragma unroll
-  for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.f;
+  for (int a = 0; a < MI; ++a)
+#pragma unroll
+    for (int b = 0; b < NJ; ++b)
+#pragma unroll
+      for (int g = 0; g < NB; ++g)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[a][b][g][e] = 0.f;
   load(0);
   put(0);
   __syncthreads();
@@ -226,29 +234,61 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(const T* __restrict__ X
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int piece = (2 * i + half) * 16;
-      const op_t a = *reinterpret_cast<const op_t*>(base + (wr * 32 + r) * kMoeRowBytes + piece);
-      const op_t b0 = *reinterpret_cast<const op_t*>(base + (AROWS + wc * 32 + r) * kMoeRowBytes + piece);
-      acc0 = moe_mfma(a, b0, acc0);
-      if (MODE == 0) {
-        const op_t b1 = *reinterpret_cast<const op_t*>(base + (AROWS + 64 + wc * 32 + r) * kMoeRowBytes + piece);
-        acc1 = moe_mfma(a, b1, acc1);
-      }
+      op_t av[MI], bv[NJ][NB];
+#pragma unroll
+      for (int a = 0; a < MI; ++a)
+        av[a] = *reinterpret_cast<const op_t*>(base + (wr * 32 * MI + 32 * a + r) * kMoeRowBytes + piece);
+#pragma unroll
+      for (int b = 0; b < NJ; ++b)
+#pragma unroll
+        for (int g = 0; g < NB; ++g)
+          bv[b][g] = *reinterpret_cast<const op_t*>(
+              base + (AROWS + g * BCOLS + wc * 32 * NJ + 32 * b + r) * kMoeRowBytes + piece);
+#pragma unroll
+      for (int a = 0; a < MI; ++a)
+#pragma unroll
+        for (int b = 0; b < NJ; ++b)
+#pragma unroll
+          for (int g = 0; g < NB; ++g) acc[a][b][g] = moe_mfma(av[a], bv[b][g], acc[a][b][g]);
     }
     if (more) put(buf ^ 1);
     __syncthreads();
   }
-  const int c = c0 + wc * 32 + r;
-  if (c >= M) return;
 #pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const int row = wr * 32 + 8 * (e / 4) + 4 * half + e % 4;
-    if (row >= count) continue;
-    const long dst = (long)sorted[start + row] * M + c;
-    if (MODE == 0)
-      reinterpret_cast<T*>(out_)[dst] = from_f32<T>(gated(acc0[e], acc1[e], act, limit, alpha));
-    else
-      reinterpret_cast<float*>(out_)[dst] = acc0[e];
+  for (int b = 0; b < NJ; ++b) {
+    const int c = c0 + wc * 32 * NJ + 32 * b + r;
+    if (c >= M) continue;
+#pragma unroll
+    for (int a = 0; a < MI; ++a)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wr * 32 * MI + 32 * a + 8 * (e / 4) + 4 * half + e % 4;
+        if (row >= count) continue;
+        const long dst = (long)sorted[start + row] * M + c;
+        if (MODE == 0)
+          reinterpret_cast<T*>(out_)[dst] = from_f32<T>(gated(acc[a][b][0][e], acc[a][b][NB - 1][e], act, limit, alpha));
+        else
+          reinterpret_cast<float*>(out_)[dst] = acc[a][b][0][e];
+      }
   }
+}
+
+template <typename T, int MODE, int MI, int NJ>
+static int launch_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
+                             int max_tiles, int top, int m, int k, int act, float limit, float alpha,
+                             hipStream_t stream) {
+  const size_t lds = (size_t)2 * (64 * MI + 64 * NJ * (MODE == 0 ? 2 : 1)) * kMoeRowBytes;
+  static int raised = 0;
+  if (lds > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)moe_expert_kernel<T, MODE, MI, NJ>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) KLLM_FAIL((int)e, "moe_expert: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    raised = 1;
+  }
+  const dim3 grid(max_tiles, ceil_div(m, 64 * NJ));
+  hipLaunchKernelGGL((moe_expert_kernel<T, MODE, MI, NJ>), grid, dim3(256), lds, stream, (const T*)x, (const T*)w, out,
+                     sorted, tiles, top, m, k, act, limit, alpha);
+  return 0;
 }
 
 // The same products for few entries (decode batches), without tiles or a plan: a workgroup takes
@@ -344,38 +384,44 @@ extern "C" int kllm_moe_route(const float* z, int nsplit, long split_stride, con
   return 0;
 }
 
-extern "C" int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int* sorted, int* tiles,
-                             hipStream_t stream) {
+extern "C" int kllm_moe_plan(const int* idx, int entries, int E, int max_tiles, int tile_rows, int* sorted,
+                             int* tiles, hipStream_t stream) {
   KLLM_REQUIRE(idx && sorted && tiles, "moe_plan: null pointer");
   KLLM_REQUIRE(entries > 0 && E > 0 && E <= 4096, "moe_plan: bad sizes entries=%d experts=%d", entries, E);
-  KLLM_REQUIRE(max_tiles >= ceil_div(entries, kMoeTileRows) + E, "moe_plan: %d tiles do not hold %d entries of %d experts",
+  KLLM_REQUIRE(tile_rows == kMoeTileRows || tile_rows == 2 * kMoeTileRows, "moe_plan: tiles of %d rows are not built",
+               tile_rows);
+  KLLM_REQUIRE(max_tiles >= ceil_div(entries, tile_rows) + E, "moe_plan: %d tiles do not hold %d entries of %d experts",
                max_tiles, entries, E);
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), stream, idx, entries, E,
-                     max_tiles, sorted, tiles);
+                     max_tiles, tile_rows, sorted, tiles);
   KLLM_CHECK_LAUNCH("moe_plan");
   return 0;
 }
 
 extern "C" int kllm_moe_expert(const void* x, const void* w, void* out, const int* sorted, const int* tiles,
-                               int max_tiles, int top, int m, int k, int mode, int act, float limit, float alpha,
-                               int dtype, hipStream_t stream) {
+                               int max_tiles, int tile_rows, int top, int m, int k, int mode, int act, float limit,
+                               float alpha, int dtype, hipStream_t stream) {
   KLLM_REQUIRE(x && w && out && sorted && tiles, "moe_expert: null pointer");
   KLLM_REQUIRE(max_tiles > 0 && top > 0 && m > 0 && k > 0, "moe_expert: bad sizes tiles=%d top=%d m=%d k=%d", max_tiles,
                top, m, k);
+  KLLM_REQUIRE(tile_rows == kMoeTileRows || tile_rows == 2 * kMoeTileRows, "moe_expert: tiles of %d rows are not built",
+               tile_rows);
   KLLM_REQUIRE(mode == 0 || mode == 1, "moe_expert: mode %d", mode);
   KLLM_REQUIRE(mode == 1 || gated_known(act), "moe_expert: unknown activation %d", act);
   KLLM_REQUIRE(dtype == DT_F32 || dtype == DT_BF16, "moe_expert: unknown dtype %d", dtype);
-  const dim3 grid(max_tiles, ceil_div(m, 64));
-  const size_t lds = (size_t)2 * (kMoeTileRows + (mode == 0 ? 128 : 64)) * kMoeRowBytes;
-#define KLLM_MOE(T, MODE)                                                                                            \
-  hipLaunchKernelGGL((moe_expert_kernel<T, MODE>), grid, dim3(256), lds, stream, (const T*)x, (const T*)w, out, sorted, \
-                     tiles, top, m, k, act, limit, alpha)
+  int rc;
+#define KLLM_MOE(T, MODE)                                                                                        \
+  rc = tile_rows == kMoeTileRows                                                                                 \
+           ? launch_moe_expert<T, MODE, 1, 1>(x, w, out, sorted, tiles, max_tiles, top, m, k, act, limit, alpha, stream) \
+           : launch_moe_expert<T, MODE, 2, MODE == 0 ? 1 : 2>(x, w, out, sorted, tiles, max_tiles, top, m, k, act, limit, \
+                                                              alpha, stream)
   if (dtype == DT_F32) {
     if (mode == 0) KLLM_MOE(float, 0); else KLLM_MOE(float, 1);
   } else {
     if (mode == 0) KLLM_MOE(bf16_t, 0); else KLLM_MOE(bf16_t, 1);
   }
 #undef KLLM_MOE
+  if (rc) return rc;
   KLLM_CHECK_LAUNCH("moe_expert");
   return 0;
 }

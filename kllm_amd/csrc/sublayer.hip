@@ -24,14 +24,41 @@ constexpr int kRowThreads = 256;
 // everything it reads (the sums' slices, the bias, the stream, the weight) is asked for before
 // the first use, so that a row costs one trip to memory (decode batches: one row, one workgroup).
 // PER == 0: rows of any length, the row's sums kept in LDS between the two passes.
+// The sums may also be those of a token's chosen experts, not yet added up (`chosen`): then
+// v = sum over the token's choices of wgt * (expert < E ? y[choice] : the feed-forward's input)
+// + the slices of delta (a shared expert's) + the bias.
+struct ChosenSums {
+  const float* y;        // [n * top][d], null: none
+  const void* xin;       // [n][d] in xin_dtype: what an identity expert hands on
+  const int* idx;        // [n][top]
+  const float* wgt;      // [n][top]
+  int top, E, xin_dtype;
+};
+
 template <typename TOUT, int PER>
 __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int nsplit, long split_stride,
-    const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps) {
+    const float* __restrict__ bias, const float* __restrict__ w, TOUT* __restrict__ out, int d, float eps,
+    const ChosenSums chosen) {
   extern __shared__ float row_lds[];      // [d] (PER == 0)
   __shared__ float red[16];
   const long r = blockIdx.x;
   float* xr = x + r * d;
+  const bool sums = delta || chosen.y;    // otherwise the stream itself is normalised
+  auto chosen_at = [&](int i) {
+    float t = 0.f;
+    for (int s = 0; s < chosen.top; ++s) {
+      const long entry = r * chosen.top + s;
+      float part;
+      if (chosen.idx[entry] < chosen.E)
+        part = chosen.y[entry * d + i];
+      else
+        part = chosen.xin_dtype == DT_BF16 ? to_f32(reinterpret_cast<const bf16_t*>(chosen.xin)[r * d + i])
+                                           : reinterpret_cast<const float*>(chosen.xin)[r * d + i];
+      t = fmaf(chosen.wgt[entry], part, t);
+    }
+    return t;
+  };
   if constexpr (PER > 0) {
     float v[PER], xv[PER], wv[PER];
 #pragma unroll
@@ -42,8 +69,10 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
       xv[j] = xr[ii];
       wv[j] = w[ii];
       float t = 0.f;
-      if (delta) {
-        for (int s = 0; s < nsplit; ++s) t += delta[s * split_stride + r * d + ii];
+      if (sums) {
+        if (chosen.y) t = chosen_at(ii);
+        if (delta)
+          for (int s = 0; s < nsplit; ++s) t += delta[s * split_stride + r * d + ii];
         if (bias) t += bias[ii];
       } else {
         t = xv[j];
@@ -59,7 +88,7 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
       const int i = threadIdx.x + kRowThreads * j;
       if (i >= d) continue;
       const float y = v[j] * rstd * wv[j];
-      const float nv = delta ? xv[j] + y : y;
+      const float nv = sums ? xv[j] + y : y;
       xr[i] = nv;
       if (out) out[r * d + i] = from_f32<TOUT>(nv);
     }
@@ -68,9 +97,10 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
   float ss = 0.f;
   for (int i = threadIdx.x; i < d; i += kRowThreads) {
     float v;
-    if (delta) {
-      v = 0.f;
-      for (int s = 0; s < nsplit; ++s) v += delta[s * split_stride + r * d + i];
+    if (sums) {
+      v = chosen.y ? chosen_at(i) : 0.f;
+      if (delta)
+        for (int s = 0; s < nsplit; ++s) v += delta[s * split_stride + r * d + i];
       if (bias) v += bias[i];
     } else {
       v = xr[i];
@@ -82,7 +112,7 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
   const float rstd = 1.f / sqrtf(total / (float)d + eps);
   for (int i = threadIdx.x; i < d; i += kRowThreads) {    // a thread reads back what it wrote itself
     const float y = row_lds[i] * rstd * w[i];
-    const float v = delta ? xr[i] + y : y;
+    const float v = sums ? xr[i] + y : y;
     xr[i] = v;
     if (out) out[r * d + i] = from_f32<TOUT>(v);
   }
@@ -192,16 +222,23 @@ using namespace kllm;
 
 extern "C" int kllm_norm_residual(float* x, const float* delta, int nsplit, long split_stride, const float* bias,
                                   const float* weight, void* out, int out_dtype, int n, int d, float eps,
-                                  hipStream_t stream) {
+                                  const float* chosen_y, const void* chosen_x, int chosen_x_dtype, const int* chosen_idx,
+                                  const float* chosen_wgt, int top, int E, hipStream_t stream) {
   KLLM_REQUIRE(x && weight, "norm_residual: null pointer");
+  KLLM_REQUIRE(!chosen_y || (chosen_x && chosen_idx && chosen_wgt && top > 0 && E >= 0 &&
+                             (chosen_x_dtype == DT_F32 || chosen_x_dtype == DT_BF16)),
+               "norm_residual: the chosen experts' sums come with their input, choices and weights");
+  ChosenSums chosen;
+  chosen.y = chosen_y; chosen.xin = chosen_x; chosen.idx = chosen_idx; chosen.wgt = chosen_wgt;
+  chosen.top = top; chosen.E = E; chosen.xin_dtype = chosen_x_dtype;
   KLLM_REQUIRE(n > 0 && d > 0 && d <= 16384, "norm_residual: bad sizes n=%d d=%d (rows of up to 16384)", n, d);
   KLLM_REQUIRE(!delta || nsplit >= 1, "norm_residual: nsplit %d", nsplit);
-  KLLM_REQUIRE(delta || !bias, "norm_residual: a bias goes with sums");
+  KLLM_REQUIRE(delta || chosen_y || !bias, "norm_residual: a bias goes with sums");
   KLLM_REQUIRE(out_dtype == DT_F32 || out_dtype == DT_BF16, "norm_residual: unknown dtype %d", out_dtype);
 #define KLLM_NR(TOUT, PER)                                                                                    \
   hipLaunchKernelGGL((norm_residual_kernel<TOUT, PER>), dim3(n), dim3(kRowThreads),                           \
                      PER ? 0 : (size_t)d * sizeof(float), stream, x, delta, nsplit, split_stride, bias, weight, \
-                     (TOUT*)out, d, eps)
+                     (TOUT*)out, d, eps, chosen)
   const bool bf = out && out_dtype == DT_BF16;
   if (d <= 4 * kRowThreads) {
     if (bf) KLLM_NR(bf16_t, 4); else KLLM_NR(float, 4);

@@ -113,14 +113,14 @@ def _declare(lib):
         "kllm_run_commands": [P, L, P, P],
         "kllm_fused_linear_max_parts": [],
         "kllm_attn_generic": [P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F, P, I, P],
-        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P],
+        "kllm_norm_residual": [P, P, I, L, P, P, P, I, I, I, F, P, P, I, P, P, I, I, P],
         "kllm_rope_tables_freq": [P, P, P, P, I, I, D, P],
         "kllm_qkv_norm_append": [P, I, L, P, P, P, I, I, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "kllm_gate_bias": [P, I, L, P, P, I, I, I, I, F, F, P],
         "kllm_moe_tile_rows": [],
         "kllm_moe_route": [P, I, L, P, I, I, I, P, P, P],
-        "kllm_moe_plan": [P, I, I, I, P, P, P],
-        "kllm_moe_expert": [P, P, P, P, P, I, I, I, I, I, I, F, F, I, P],
+        "kllm_moe_plan": [P, I, I, I, I, P, P, P],
+        "kllm_moe_expert": [P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "kllm_moe_expert_rows": [P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "kllm_moe_combine": [P, P, P, P, P, I, L, P, I, I, I, I, I, P],
         "kllm_sample": [P, P, P, P, I, I, P],
@@ -1352,11 +1352,28 @@ def delta_out(o, gate, weight, eps, out, heads, head_dim):
 
 # ----------------------------------------------------------------------------- norm behind the sub-layer, rotation then unit norm, routed experts
 
+class ChosenSums:
+    """What a routed feed-forward leaves for the norm behind it to add up: per token the weighted
+    sum over its choices of ``y`` [n * top, d] (float32), or of ``xin`` [n, d] where the chosen
+    expert is an identity (``idx`` >= ``experts``), plus the slices of ``shared`` (or None)."""
+
+    def __init__(self, y, xin, idx, wgt, experts, shared=None):
+        self.y, self.xin, self.idx, self.wgt, self.experts, self.shared = y, xin, idx, wgt, int(experts), shared
+
+
 def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
-    """x [n, d] float32 in place.  With ``delta`` (float32 [n, d] or [nsplit, n, d]; ``bias`` [d] is
-    added to it): x += weight * N(delta + bias); without: x = weight * N(x), where N divides a
-    row by sqrt(mean of its squares + eps).  ``out`` [n, d] receives the new x in its own dtype."""
+    """x [n, d] float32 in place.  With ``delta`` (float32 [n, d] or [nsplit, n, d], or a
+    ``ChosenSums``; ``bias`` [d] is added to it): x += weight * N(delta + bias); without: x =
+    weight * N(x), where N divides a row by sqrt(mean of its squares + eps).  ``out`` [n, d]
+    receives the new x in its own dtype."""
     n, d = x.shape
+    chosen = None
+    if isinstance(delta, ChosenSums):
+        chosen, delta = delta, delta.shared
+        top = chosen.idx.shape[1]
+        if (tuple(chosen.y.shape) != (n * top, d) or tuple(chosen.xin.shape) != (n, d)
+                or tuple(chosen.wgt.shape) != (n, top)):
+            raise KernelError("norm_residual: the chosen experts' sums do not fit")
     nsplit, stride = (1, 0) if delta is None else _splits(delta, n, d, "norm_residual")
     if weight.numel() != d or (bias is not None and bias.numel() != d) or (out is not None and tuple(out.shape) != (n, d)):
         raise KernelError("norm_residual: weight, bias or output does not fit")
@@ -1364,7 +1381,12 @@ def norm_residual(x, weight, delta=None, bias=None, out=None, eps=0.0):
     _launch("kllm_norm_residual", "norm_residual", _ptr(x, "norm_residual x", F32),
             _ptr(delta, "norm_residual delta", F32, True), nsplit, stride, _ptr(bias, "norm_residual bias", F32, True),
             _ptr(weight, "norm_residual weight", F32), _ptr(out, "norm_residual out", None, True),
-            dtype_code(out.dtype) if out is not None else DT_F32, n, d, float(eps), _stream())
+            dtype_code(out.dtype) if out is not None else DT_F32, n, d, float(eps),
+            _ptr(chosen.y, "norm_residual y", F32) if chosen else 0, _ptr(chosen.xin, "norm_residual xin") if chosen else 0,
+            dtype_code(chosen.xin.dtype) if chosen else DT_F32,
+            _ptr(chosen.idx, "norm_residual idx", torch.int32) if chosen else 0,
+            _ptr(chosen.wgt, "norm_residual wgt", F32) if chosen else 0, chosen.idx.shape[1] if chosen else 0,
+            chosen.experts if chosen else 0, _stream())
 
 
 def rope_tables_freq(cos, sin, positions, freq, factor=1.0):
@@ -1426,9 +1448,16 @@ def moe_tile_rows() -> int:
     return limit("moe_tile_rows")
 
 
-def moe_max_tiles(entries, experts) -> int:
-    """Tiles that always hold ``entries`` (token, choice) pairs of ``experts`` experts."""
-    return -(-entries // moe_tile_rows()) + experts
+def moe_max_tiles(entries, experts, tile_rows=None) -> int:
+    """Tiles of ``tile_rows`` rows that always hold ``entries`` (token, choice) pairs of ``experts`` experts."""
+    return -(-entries // (tile_rows or moe_tile_rows())) + experts
+
+
+def moe_best_tile_rows(entries, experts) -> int:
+    """Rows of a tile for this many entries: the large tiles (twice ``moe_tile_rows()``, as many
+    columns) from where an expert's share fills one, the small ones below."""
+    small = moe_tile_rows()
+    return 2 * small if entries >= 2 * small * experts else small
 
 
 def moe_route(z, correction, idx, wgt):
@@ -1443,15 +1472,16 @@ def moe_route(z, correction, idx, wgt):
             _ptr(idx, "moe_route idx", torch.int32), _ptr(wgt, "moe_route wgt", torch.float32), _stream())
 
 
-def moe_plan(idx, experts, sorted_entries, tiles):
+def moe_plan(idx, experts, sorted_entries, tiles, tile_rows=None):
     entries = idx.numel()
+    tile_rows = int(tile_rows or moe_tile_rows())
     if sorted_entries.numel() < entries or tiles.dim() != 2 or tiles.shape[1] != 3:
         raise KernelError("moe_plan: outputs do not fit")
     _launch("kllm_moe_plan", "moe_plan", _ptr(idx, "moe_plan idx", torch.int32), entries, int(experts), tiles.shape[0],
-            _ptr(sorted_entries, "moe_plan sorted", torch.int32), _ptr(tiles, "moe_plan tiles", torch.int32), _stream())
+            tile_rows, _ptr(sorted_entries, "moe_plan sorted", torch.int32), _ptr(tiles, "moe_plan tiles", torch.int32), _stream())
 
 
-def moe_expert(x, w, out, sorted_entries, tiles, top, mode, act=ACT_SILU, limit=0.0, alpha=1.0):
+def moe_expert(x, w, out, sorted_entries, tiles, top, mode, act=ACT_SILU, limit=0.0, alpha=1.0, tile_rows=None):
     """mode 0: x [tokens, k], w [E, 2m, k] -> out [tokens * top, m] gated, in x's dtype;
     mode 1: x [tokens * top, k], w [E, m, k] -> out [tokens * top, m] float32."""
     k = x.shape[1]
@@ -1462,8 +1492,8 @@ def moe_expert(x, w, out, sorted_entries, tiles, top, mode, act=ACT_SILU, limit=
         raise KernelError(f"moe_expert: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
     _launch("kllm_moe_expert", "moe_expert", _ptr(x, "moe_expert x"), _ptr(w, "moe_expert w"), _ptr(out, "moe_expert out"),
             _ptr(sorted_entries, "moe_expert sorted", torch.int32), _ptr(tiles, "moe_expert tiles", torch.int32),
-            tiles.shape[0], int(top), m, k, int(mode), int(act), float(limit), float(alpha), dtype_code(x.dtype),
-            _stream())
+            tiles.shape[0], int(tile_rows or moe_tile_rows()), int(top), m, k, int(mode), int(act), float(limit),
+            float(alpha), dtype_code(x.dtype), _stream())
 
 
 MOE_ROWS_BEST_ENTRIES = 16     # (token, choice) pairs up to which the entry-by-entry products beat the tiles

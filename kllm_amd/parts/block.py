@@ -215,7 +215,9 @@ class SublayerNormBlock(Part):
                         eps=self.norm_mixer.eps)
         if self.feed_forward is not None:
             xin = stream_copy(ctx, x)
-            delta = call_part(self.feed_forward, self.feed_forward.forward, ctx, xin)
+            # a routed feed-forward's weighted sum over the chosen experts is taken in the norm's launch
+            more = {"sums_ok": True} if getattr(self.feed_forward, "leaves_chosen_sums", False) else {}
+            delta = call_part(self.feed_forward, self.feed_forward.forward, ctx, xin, **more)
             K.norm_residual(x, self.norm_ff.weight, delta, bias=getattr(self.feed_forward, "out_bias", None), out=out,
                             eps=self.norm_ff.eps)
         return x, None

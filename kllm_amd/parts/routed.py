@@ -111,7 +111,11 @@ class RoutedExperts(Part):
             total += 6.0 * tokens * d * self.shared_intermediate
         return total
 
-    def forward(self, ctx, xn):
+    # The weighted sum over a token's choices can be left to a norm that adds it up while it
+    # normalises (``sums_ok``: the caller takes a ``kernels.ChosenSums``).
+    leaves_chosen_sums = True
+
+    def forward(self, ctx, xn, sums_ok=False):
         n, d, top, f = xn.shape[0], self.hidden, self.top, self.intermediate
         dtype = self.runtime.dtype
         z = decode_linear(ctx, xn, self.w_router, "moe.z", self._tiled.get("router"))
@@ -125,16 +129,19 @@ class RoutedExperts(Part):
             K.moe_expert_rows(xn, self.w_gu, h, idx, self.experts, 0, self.act, self.limit, self.alpha)
             K.moe_expert_rows(h, self.w_down, y, idx, self.experts, 1)
         else:
-            tiles = ctx.buf("moe.tiles", (K.moe_max_tiles(n * top, self.experts), 3), torch.int32)
+            rows = K.moe_best_tile_rows(n * top, self.experts)
+            tiles = ctx.buf("moe.tiles", (K.moe_max_tiles(n * top, self.experts, rows), 3), torch.int32)
             order = ctx.buf("moe.sorted", (n * top,), torch.int32)
-            K.moe_plan(idx, self.experts, order, tiles)
-            K.moe_expert(xn, self.w_gu, h, order, tiles, top, 0, self.act, self.limit, self.alpha)
-            K.moe_expert(h, self.w_down, y, order, tiles, top, 1)
+            K.moe_plan(idx, self.experts, order, tiles, rows)
+            K.moe_expert(xn, self.w_gu, h, order, tiles, top, 0, self.act, self.limit, self.alpha, tile_rows=rows)
+            K.moe_expert(h, self.w_down, y, order, tiles, top, 1, tile_rows=rows)
         shared = None
         if self.shared_intermediate:
             hs = gated_hidden(ctx, xn, self.w_shared_gu, self.shared_intermediate, "moe.shared",
                               self._tiled.get("shared_gu"), None, self.act, self.shared_limit, self.alpha)
             shared = decode_linear(ctx, hs, self.w_shared_down, "moe.shared.down", self._tiled.get("shared_down"))
+        if sums_ok:
+            return K.ChosenSums(y, xn, idx, wgt, self.experts, shared)
         out = ctx.buf("moe.out", (n, d), torch.float32)
         K.moe_combine(y, xn, idx, wgt, out, self.experts, shared)
         return out

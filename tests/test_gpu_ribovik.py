@@ -286,25 +286,33 @@ def test_routed_experts_against_the_plain_mixture(n, d, E, ident, top, f, shared
     if n >= 70:     # the corrections did change the choice
         plain_top = torch.topk(torch.softmax(h64 @ w64["m.router"].T, -1), top).indices
         assert not torch.equal(idx_want.sort(1).values, plain_top.sort(1).values)
-    tiles = torch.full((K.moe_max_tiles(n * top, E), 3), -7, device="cuda", dtype=torch.int32)
-    order = torch.full((n * top,), -1, device="cuda", dtype=torch.int32)
-    K.moe_plan(idx, E, order, tiles)
-    real = int((idx.cpu() < E).sum())
-    assert sorted(order.cpu().tolist()[:real]) == sorted(torch.nonzero(idx.cpu().flatten() < E).flatten().tolist())
-    assert int(tiles.cpu()[:, 2].sum()) == real and int(tiles.cpu()[:, 2].max()) <= K.moe_tile_rows()
     w_gu = dev(torch.stack([torch.cat([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(E)]), dt).contiguous()
     w_down = dev(torch.stack([w[f"e{e}.down"] for e in range(E)]), dt).contiguous()
-    hh = torch.full((n * top, f), float("nan"), device="cuda", dtype=dt)
-    K.moe_expert(hd, w_gu, hh, order, tiles, top, 0, K.GATE_CLAMPED_SWISH, 1.2, 1.702)
-    y = torch.full((n * top, d), float("nan"), device="cuda")
-    K.moe_expert(hh, w_down, y, order, tiles, top, 1)
     sh = None
     if shared:
         sh = P.clamped_expert(h64, w64, "m.shared", 0.7)
         sh = dev(torch.stack([0.5 * sh, 0.5 * sh]).float())
-    out = torch.empty(n, d, device="cuda")
-    K.moe_combine(y, hd, idx, wgt, out, E, sh)
-    assert rel(out.cpu(), want) < (2e-6 if dtype == "float32" else 6e-3)
+    real = int((idx.cpu() < E).sum())
+    for rows in (K.moe_tile_rows(), 2 * K.moe_tile_rows()):          # both shapes of tiles
+        tiles = torch.full((K.moe_max_tiles(n * top, E, rows), 3), -7, device="cuda", dtype=torch.int32)
+        order = torch.full((n * top,), -1, device="cuda", dtype=torch.int32)
+        K.moe_plan(idx, E, order, tiles, rows)
+        assert sorted(order.cpu().tolist()[:real]) == sorted(torch.nonzero(idx.cpu().flatten() < E).flatten().tolist())
+        assert int(tiles.cpu()[:, 2].sum()) == real and int(tiles.cpu()[:, 2].max()) <= rows
+        hh = torch.full((n * top, f), float("nan"), device="cuda", dtype=dt)
+        K.moe_expert(hd, w_gu, hh, order, tiles, top, 0, K.GATE_CLAMPED_SWISH, 1.2, 1.702, tile_rows=rows)
+        y = torch.full((n * top, d), float("nan"), device="cuda")
+        K.moe_expert(hh, w_down, y, order, tiles, top, 1, tile_rows=rows)
+        out = torch.empty(n, d, device="cuda")
+        K.moe_combine(y, hd, idx, wgt, out, E, sh)
+        assert rel(out.cpu(), want) < (2e-6 if dtype == "float32" else 6e-3), rows
+    # the norm behind the layer takes the weighted sum in its own launch
+    xs, wn = torch.randn(n, d, generator=g), 1 + 0.2 * torch.randn(d, generator=g)
+    xd, ob = dev(xs.clone()), torch.empty(n, d, device="cuda", dtype=dt)
+    K.norm_residual(xd, dev(wn), K.ChosenSums(y, hd, idx, wgt, E, sh), out=ob, eps=1e-5)
+    after = xs.double() + P.rms_norm(want, wn.double(), 1e-5)
+    assert rel(xd.cpu(), after) < (2e-6 if dtype == "float32" else 6e-3)
+    assert rel(ob.float().cpu(), after) < (2e-6 if dtype == "float32" else 8e-3)
     if n * top <= 64:       # the same entry by entry, as decode batches run it
         hh.fill_(float("nan"))
         y.fill_(float("nan"))
