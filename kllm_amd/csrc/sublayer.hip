@@ -60,25 +60,56 @@ __global__ __launch_bounds__(kRowThreads) void norm_residual_kernel(
     return t;
   };
   if constexpr (PER > 0) {
+    // Loops over slices and choices stand outside the loop over a thread's elements, whose
+    // loads then go out together (a load behind a loop of unknown length is waited for at once).
     float v[PER], xv[PER], wv[PER];
+    int at[PER];
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int i = threadIdx.x + kRowThreads * j;
-      const bool ok = i < d;
-      const int ii = ok ? i : 0;
-      xv[j] = xr[ii];
-      wv[j] = w[ii];
-      float t = 0.f;
-      if (sums) {
-        if (chosen.y) t = chosen_at(ii);
-        if (delta)
-          for (int s = 0; s < nsplit; ++s) t += delta[s * split_stride + r * d + ii];
-        if (bias) t += bias[ii];
-      } else {
-        t = xv[j];
-      }
-      v[j] = ok ? t : 0.f;
+      at[j] = i < d ? i : 0;
+      xv[j] = xr[at[j]];
+      wv[j] = w[at[j]];
+      v[j] = 0.f;
     }
+    if (sums) {
+      if (chosen.y) {
+        for (int s = 0; s < chosen.top; ++s) {
+          const long entry = r * chosen.top + s;
+          const float weight = chosen.wgt[entry];
+          if (chosen.idx[entry] < chosen.E) {
+            const float* src = chosen.y + entry * d;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) v[j] = fmaf(weight, src[at[j]], v[j]);
+          } else if (chosen.xin_dtype == DT_BF16) {
+            const bf16_t* src = reinterpret_cast<const bf16_t*>(chosen.xin) + r * d;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) v[j] = fmaf(weight, to_f32(src[at[j]]), v[j]);
+          } else {
+            const float* src = reinterpret_cast<const float*>(chosen.xin) + r * d;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) v[j] = fmaf(weight, src[at[j]], v[j]);
+          }
+        }
+      }
+      if (delta) {
+        for (int s = 0; s < nsplit; ++s) {
+          const float* src = delta + s * split_stride + r * d;
+#pragma unroll
+          for (int j = 0; j < PER; ++j) v[j] += src[at[j]];
+        }
+      }
+      if (bias) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) v[j] += bias[at[j]];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < PER; ++j) v[j] = xv[j];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (threadIdx.x + kRowThreads * j >= d) v[j] = 0.f;
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < PER; ++j) ss = fmaf(v[j], v[j], ss);
