@@ -181,15 +181,30 @@ __global__ __launch_bounds__(256) void qkv_norm_append_kernel(
   const int slot = pos % page_size;
   const long kblock = (long)page_size * dk, vblock = (long)page_size * dv;
   T* page_base = cache + page * KV * (kblock + vblock);
-  auto sum_at = [&](long col) {
-    float v = 0.f;
-    for (int s = 0; s < nsplit; ++s) v += in[s * split_stride + col];
-    return bias ? v + bias[col] : v;
-  };
+  // Loops over the sums' slices stand outside the loops over a lane's elements, whose loads then
+  // go out together.
   if (item >= H + KV) {     // a value head: stored with the slot as the fast index
     const int h = item - H - KV;
+    const long vcol = (long)(H + KV) * dk + h * dv;
+    float v[4];
+    int col[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = lane + kWave * r;
+      col[r] = j < dv ? j : 0;
+      v[r] = 0.f;
+    }
+    for (int s = 0; s < nsplit; ++s) {
+      const float* src = in + s * split_stride + vcol;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] += src[col[r]];
+    }
     T* vdst = page_base + KV * kblock + h * vblock + slot;
-    for (int j = lane; j < dv; j += kWave) vdst[(long)j * page_size] = from_f32<T>(sum_at((long)(H + KV) * dk + h * dv + j));
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = lane + kWave * r;
+      if (j < dv) vdst[(long)j * page_size] = from_f32<T>(bias ? v[r] + bias[vcol + j] : v[r]);
+    }
     return;
   }
   const bool is_q = item < H;
@@ -198,21 +213,36 @@ __global__ __launch_bounds__(256) void qkv_norm_append_kernel(
   const int pairs = dk / 2, rhalf = rot / 2;
   float ra[2], rb[2];
   int ea[2], eb[2];
+  float a[2] = {0.f, 0.f}, b[2] = {0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int j = lane + kWave * r;
+    // the two elements of this pair: one that turns, or two neighbours that pass through
+    ea[r] = j >= pairs ? 0 : j < rhalf ? (interleaved ? 2 * j : j) : rot + 2 * (j - rhalf);
+    eb[r] = j >= pairs ? 0 : j < rhalf ? (interleaved ? 2 * j + 1 : j + rhalf) : ea[r] + 1;
+  }
+  for (int s = 0; s < nsplit; ++s) {
+    const float* src = in + s * split_stride + base;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      a[r] += src[ea[r]];
+      b[r] += src[eb[r]];
+    }
+  }
   float ss = 0.f;
 #pragma unroll
   for (int r = 0; r < 2; ++r) {
     const int j = lane + kWave * r;
     ra[r] = rb[r] = 0.f;
-    ea[r] = eb[r] = 0;
     if (j >= pairs) continue;
+    if (bias) {
+      a[r] += bias[base + ea[r]];
+      b[r] += bias[base + eb[r]];
+    }
     const bool turns = cos_t && j < rhalf;
-    // the two elements of this pair: one that turns, or two neighbours that pass through
-    ea[r] = j < rhalf ? (interleaved ? 2 * j : j) : rot + 2 * (j - rhalf);
-    eb[r] = j < rhalf ? (interleaved ? 2 * j + 1 : j + rhalf) : ea[r] + 1;
-    const float a = sum_at(base + ea[r]), b = sum_at(base + eb[r]);
-    const float c = turns ? cos_t[t * rhalf + j] : 1.f, s = turns ? sin_t[t * rhalf + j] : 0.f;
-    ra[r] = a * c - b * s;
-    rb[r] = b * c + a * s;
+    const float c = turns ? cos_t[t * rhalf + j] : 1.f, sn = turns ? sin_t[t * rhalf + j] : 0.f;
+    ra[r] = a[r] * c - b[r] * sn;
+    rb[r] = b[r] * c + a[r] * sn;
     ss += ra[r] * ra[r] + rb[r] * rb[r];
   }
   float rstd = 1.f;

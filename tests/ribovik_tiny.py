@@ -71,9 +71,9 @@ CONFIGS = {
         attn(6, 3, 16, rot=16, base=1000.0, scaling=(1.5, 32, 8.0, 4.0), chunk=16, mlp=dense(56)),
         attn(6, 3, 16, rot=16, base=1000.0, scaling=(1.5, 32, 8.0, 4.0), chunk=16, mlp=dense(56))]),
     "R6": _cfg(150, 160, 1e-6, [
-        attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 32.0, 1.0), chunk=100,
+        attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 24.0, 1.5), chunk=100,
              mlp=moe(4, 2, 3, 40, 0.3, shared=(64, 0.5))),
-        attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 32.0, 1.0), chunk=100, mlp=dense(72))]),
+        attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 24.0, 1.5), chunk=100, mlp=dense(72))]),
 }
 
 
