@@ -126,7 +126,8 @@ def spans_context(lens, starts_pos):
 
 ATTN_CASES = [  # H, KV, dk, dv, rotated, chunk
     (4, 2, 32, 32, 16, 24), (4, 1, 64, 64, 64, 40), (8, 1, 32, 32, 0, 0), (2, 2, 128, 128, 64, 100),
-    (6, 3, 24, 24, 12, 7), (5, 5, 20, 12, 10, 33), (10, 2, 80, 80, 32, 16), (4, 1, 64, 32, 32, 64), (12, 4, 16, 16, 16, 50)]
+    (6, 3, 24, 24, 12, 7), (5, 5, 20, 12, 10, 33), (10, 2, 80, 80, 32, 16), (4, 1, 64, 32, 32, 64), (12, 4, 16, 16, 16, 50), (6, 2, 48, 48, 24, 20),
+    (34, 1, 32, 32, 8, 30)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -255,7 +256,7 @@ def test_attention_kernels_at_the_edges_of_chunks_with_a_sink(H, KV, dk, dv, rot
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n", [1, 5, 70, 300])
 @pytest.mark.parametrize("d,E,ident,top,f,shared", [(64, 6, 2, 2, 48, 40), (50, 3, 1, 2, 22, 18), (128, 4, 0, 1, 32, None),
-                                                    (72, 2, 3, 4, 24, 16), (256, 40, 0, 6, 64, None)])
+                                                    (72, 2, 3, 4, 24, 16), (256, 40, 0, 6, 64, None), (64, 70, 3, 5, 16, None)])
 def test_routed_experts_against_the_plain_mixture(n, d, E, ident, top, f, shared, dtype):
     """The routed feed-forward's kernels in the order the part launches them.  Both sides get the
     same input and weights (rounded to the storage type), so the choice of experts rests on
