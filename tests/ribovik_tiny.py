@@ -15,6 +15,9 @@ R5: heads of 16 that turn whole, chunks of 16 (the page), stretched by 1.5 with 
     layers only, another eps.
 R6: heads of 96 of which 64 turn, ten heads on two KV heads, chunks of 100, experts whose limit
     clamps often, top 3 of 4 + 2.
+R7: every layer unlike the others: heads of 32, 16 and 64, values of their own width on one layer,
+    chunks of 12 and 30 and none, rotation whole, partial and none, two different mixtures, a layer
+    without feed-forward; the first and the last layer alike.
 """
 
 import json
@@ -74,6 +77,11 @@ CONFIGS = {
         attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 24.0, 1.5), chunk=100,
              mlp=moe(4, 2, 3, 40, 0.3, shared=(64, 0.5))),
         attn(10, 2, 96, rot=64, base=100000.0, scaling=(8.0, 128, 24.0, 1.5), chunk=100, mlp=dense(72))]),
+    "R7": _cfg(70, 96, 1e-5, [
+        attn(4, 2, 32, rot=32, chunk=12, mlp=dense(64)),
+        attn(6, 1, 16, rot=8, base=777.0, scaling=(3.0, 48, 12.0, 2.0), chunk=30, mlp=moe(5, 1, 2, 24, 2.5, shared=(32, 1.25))),
+        attn(2, 2, 64, vdim=48),
+        attn(4, 2, 32, rot=32, chunk=12, mlp=moe(3, 2, 3, 40, 0.8))]),
 }
 
 

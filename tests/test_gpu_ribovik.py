@@ -377,7 +377,7 @@ def compare(rows, want, dtype, requests):
 
 
 CASES = [("R1", [1, 5, 33, 130]), ("R2", [2, 17, 140]), ("R3", [3, 64, 65, 150]), ("R4", [90, 31]), ("R5", [49, 80, 16, 17]),
-         ("R6", [210, 99, 101])]
+         ("R6", [210, 99, 101]), ("R7", [75, 3, 128])]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
